@@ -1,0 +1,89 @@
+/*
+ * C ABI of libonebitmul for MI355X (gfx950): one-bit 2:4 sparse GEMM  D = alpha * A * B + beta * C.
+ *
+ * Drop-in for the reference header include/onebit_sparse_tensor.h (one declaration, line 5) and its
+ * implementation csrc/kernel_lib.cu:23-97. Plain pointers and ints only; no runtime headers are needed
+ * to call it. All pointers are DEVICE pointers unless stated otherwise.
+ *
+ * Operand formats (identical to the reference):
+ *   a  one bit per kept value of A, (m x k/2) column-major with packed stride m, LSB first:
+ *      bit (r, j) = bit (r + j*m) % 8 of byte (r + j*m) / 8; 1 -> +1.0, 0 -> -1.0
+ *      (csrc/kernel_lib.cu:28,37; csrc/kernel.h:13-14; csrc/warp.h:41-50; written by
+ *      onebit_sparse_mul/__init__.py:139-143 as a (k/2, m/8) uint8 tensor)
+ *   e  int16 metadata, m x k/16 elements, nibble g of an element = idx0 | idx1 << 2 of dense group g,
+ *      stored in the reordered layout of onebit_sparse_mul/_semi_structured_conversions.py:21-48,173-177
+ *      (csrc/kernel_lib.cu:41)
+ *   b  fp16, (k x n) row-major, packed stride n (csrc/kernel_lib.cu:38)
+ *   c  (m x n) row-major source, d  (m x n) row-major destination (csrc/kernel_lib.cu:39-40)
+ * Shape constraints: m % 64 == 0, k % 32 == 0 (where the reference metadata layout is a bijection),
+ * n >= 1. Work is enqueued on a HIP stream and the call returns without synchronising, as the reference
+ * does (csrc/kernel_lib.cu:86).
+ */
+#ifndef ONEBIT_SPARSE_TENSOR_H_
+#define ONEBIT_SPARSE_TENSOR_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* dtype codes for c / d */
+#define ONEBIT_DTYPE_F32 0
+#define ONEBIT_DTYPE_F16 1
+
+/* metadata layouts of e */
+#define ONEBIT_META_REFERENCE 0 /* onebit_sparse_mul/_semi_structured_conversions.py:21-48 (default) */
+#define ONEBIT_META_CUTLASS   1 /* CUTLASS reorder_meta (tests/unit/warp_test.h:377-379) */
+#define ONEBIT_META_LOGICAL   2 /* plain row-major (m, k/16) */
+
+/* status codes of the int-returning entry points */
+#define ONEBIT_OK             0
+#define ONEBIT_ERR_ARGUMENT   1 /* null pointer, unsupported shape / dtype / layout */
+#define ONEBIT_ERR_HIP        2 /* a HIP runtime call failed (no device, launch failure, out of memory) */
+
+/*
+ * Replaces: void onebit_sparse_matmul(void*,void*,void*,void*,void*,int,int,int)
+ *           include/onebit_sparse_tensor.h:5, csrc/kernel_lib.cu:23-97.
+ * d = 1 * A * b + 0 * c with fp32 c/d (csrc/kernel.h:17-18, csrc/kernel_lib.cu:60-61), metadata in the
+ * reference layout, enqueued on the default stream. c is not read (beta = 0) and may equal d, as the torch
+ * binding passes it (onebit_sparse_mul/torch_kernel_cuda.cpp:23-24). On any error it prints one line to
+ * stderr and calls exit(EXIT_FAILURE), which is the reference's error convention (csrc/kernel_lib.cu:11-20).
+ */
+void onebit_sparse_matmul(void *a, void *b, void *c, void *d, void *e, int m, int n, int k);
+
+/*
+ * Extended form of the entry point above (same operands; csrc/kernel_lib.cu:23-97 with the values it
+ * hard-codes at :60-62 and the dtypes of csrc/kernel.h:17-18 turned into arguments): alpha/beta epilogue
+ * (csrc/kernel.h:27-31), fp16 or fp32 c and d, metadata layout, explicit stream (hipStream_t passed as
+ * void*, NULL = default stream). Returns a status code and never exits.
+ * The reordered copy of (a, e) is written to a library-owned per-device workspace on every call, so calls
+ * that overlap on different streams of one device must use the prepared form below instead.
+ */
+int onebit_sparse_matmul_ex(const void *a, const void *b, const void *c, void *d, const void *e, int m, int n, int k,
+                            float alpha, float beta, int c_dtype, int d_dtype, int meta_layout, void *stream);
+
+/*
+ * Prepared-operand form: the weight side (a, e) is reordered once into a caller-owned device buffer and
+ * reused by every later product. Replaces the host-side metadata reordering that the reference does in
+ * Python before the call (onebit_sparse_mul/_semi_structured_conversions.py:171-177) and that CUTLASS
+ * does with reorder_meta (tests/unit/warp_test.h:377-379).
+ */
+size_t onebit_sparse_prepared_bytes(int m, int k);
+int onebit_sparse_prepare(const void *a, const void *e, int m, int k, int meta_layout, void *prepared, void *stream);
+int onebit_sparse_matmul_prepared(const void *prepared, const void *b, const void *c, void *d, int m, int n, int k,
+                                  float alpha, float beta, int c_dtype, int d_dtype, void *stream);
+
+/* Message of the last failure on the calling thread ("" if none). Host pointer, valid until the next call. */
+const char *onebit_sparse_last_error(void);
+
+/* Tuning / test hooks: force a tile configuration of the main kernel (-1 = automatic) and choose whether
+ * shapes with n <= 32 use the split-K kernel (1, default) or the main kernel (0). Process-wide. */
+void onebit_sparse_set_tile_config(int tile_config);
+void onebit_sparse_set_skinny_enabled(int enabled);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* ONEBIT_SPARSE_TENSOR_H_ */

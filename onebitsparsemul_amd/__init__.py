@@ -1,0 +1,158 @@
+"""onebitsparsemul_amd - one-bit 2:4 sparse GEMM for MI355X (gfx950).
+
+Python surface of the reference package ``onebit_sparse_mul`` (onebit_sparse_mul/__init__.py:12-145) on top
+of libonebitmul.so: same callables, same argument meaning, intended semantics where the reference's own code
+is inconsistent (result allocated on the operands' device, metadata passed in the binding's argument order,
+``y = x @ W.T`` in the linear layer). GPU work always goes through the HIP library; nothing falls back to a
+host computation.
+"""
+import torch
+import torch.nn as nn
+
+from . import _native
+from ._semi_structured_conversions import (
+    mask_creator,
+    sparse_semi_structured_from_dense_cutlass,
+    sparse_semi_structured_to_dense_cutlass,
+)
+
+__all__ = [
+    "cuda_binary_mul", "cuda_binary_mul_", "binary_quant", "pack_binary", "unpack_binary", "dequant_desparse_tile",
+    "py_binary_gemm", "BinaryLinear_2_4", "PreparedWeight", "mask_creator", "sparse_semi_structured_from_dense_cutlass",
+    "sparse_semi_structured_to_dense_cutlass",
+]
+
+
+def _binding():
+    """The compiled torch binding `onebit_sparse_cuda` (reference: onebit_sparse_mul/torch_kernel_cuda.cpp)."""
+    from . import onebit_sparse_cuda  # noqa: PLC0415  (compiled module, built in-tree)
+    return onebit_sparse_cuda
+
+
+def _problem_shape(A, B, meta):
+    m, k = meta.shape[0], meta.shape[1] * 16
+    if A.dtype != torch.uint8 or A.numel() != m * k // 16:
+        raise ValueError(f"A must be uint8 with m*k/16 = {m * k // 16} bytes (shape (k/2, m/8)), got {tuple(A.shape)}")
+    if B.dim() != 2 or B.shape[0] != k:
+        raise ValueError(f"B must have shape (k={k}, n), got {tuple(B.shape)}")
+    return m, B.shape[1], k
+
+
+def cuda_binary_mul(A, B, meta):
+    """C = W @ B with W the one-bit 2:4 weight stored as (A bits, meta); returns fp32 (m, n) on B's device.
+    Reference: onebit_sparse_mul/__init__.py:12-15."""
+    m, n, _ = _problem_shape(A, B, meta)
+    C = torch.empty((m, n), dtype=torch.float32, device=B.device)
+    _binding().onebit_mul(A, B, meta, C)
+    return C
+
+
+def cuda_binary_mul_(A, B, C, meta):
+    """In-place form: writes into C (fp32 or fp16, (m, n)). Reference: onebit_sparse_mul/__init__.py:17-19."""
+    _binding().onebit_mul(A, B, meta, C)
+    return C
+
+
+def binary_quant(tensor):
+    """value > 0 -> 1, else 0. Reference: onebit_sparse_mul/__init__.py:22-23."""
+    return (tensor > 0).to(torch.int64)
+
+
+def pack_binary(tensor):
+    """(rows, cols) of 0/1 -> (rows, cols/8) uint8; element 8c+i of a row is bit i of byte c.
+    Reference: onebit_sparse_mul/__init__.py:25-34."""
+    rows, cols = tensor.shape
+    if cols % 8:
+        raise ValueError("last dimension must be a multiple of 8")
+    weights = (1 << torch.arange(8, device=tensor.device, dtype=torch.int64))
+    return (tensor.reshape(rows, cols // 8, 8).to(torch.int64) * weights).sum(-1).to(torch.uint8)
+
+
+def unpack_binary(packed_tensor):
+    """Inverse of pack_binary; returns uint8 0/1. Reference: onebit_sparse_mul/__init__.py:36-45."""
+    rows, pcols = packed_tensor.shape
+    shifts = torch.arange(8, device=packed_tensor.device, dtype=torch.int64)
+    bits = (packed_tensor.to(torch.int64)[..., None] >> shifts) & 1
+    return bits.reshape(rows, pcols * 8).to(torch.uint8)
+
+
+def dequant_desparse_tile(packed_sparse_tile, meta_tile):
+    """(k/2, m/8) packed bits + (m, k/16) reordered metadata -> dense (m, k) weight with values in {-1, 0, +1}.
+    Reference: onebit_sparse_mul/__init__.py:47-65 (whose shapes do not compose; this is the intended result)."""
+    bits = unpack_binary(packed_sparse_tile).T.contiguous()  # (m, k/2)
+    values = torch.where(bits == 1, 1, -1).to(torch.int32)
+    return sparse_semi_structured_to_dense_cutlass(values, meta_tile)
+
+
+def py_binary_gemm(x, packed_sparse_tensor, sparse_meta):
+    """Host check: x (batch, k) @ W.T with W = dequant_desparse_tile(...), as torch.matmul on the dense weight.
+    Reference: onebit_sparse_mul/__init__.py:67-97."""
+    if packed_sparse_tensor.dtype != torch.uint8:
+        raise ValueError("packed_sparse_tensor must be `torch.uint8`")
+    if sparse_meta.dtype != torch.int16:
+        raise ValueError("Sparse Meta must be `torch.int16`")
+    if packed_sparse_tensor.shape[0] * 2 != x.shape[1]:
+        raise ValueError("x.shape[1] must equal 2 * packed_sparse_tensor.shape[0] (the weight's in-features)")
+    dense = dequant_desparse_tile(packed_sparse_tensor, sparse_meta)
+    return torch.matmul(x, dense.to(x.dtype).T)
+
+
+class PreparedWeight:
+    """A packed weight reordered once for the gfx950 kernels (see include/onebit_sparse_tensor.h)."""
+
+    def __init__(self, packed_binary_sparse, meta, layout=_native.META_REFERENCE):
+        self.m = meta.shape[0]
+        self.k = meta.shape[1] * 16
+        self.buffer = _native.prepare(packed_binary_sparse, meta, self.m, self.k, layout)
+
+    def matmul(self, b, out=None, c=None, alpha=1.0, beta=0.0, out_dtype=torch.float16):
+        n = b.shape[1]
+        if out is None:
+            out = torch.empty((self.m, n), dtype=out_dtype, device=b.device)
+        return _native.matmul_prepared(self.buffer, b, out, self.m, n, self.k, c=c, alpha=alpha, beta=beta)
+
+
+class BinaryLinear_2_4(nn.Module):
+    """1-bit 2:4 sparse linear layer without bias: y = x @ W.T, W (outfeatures, infeatures) stored at 1.5 bits
+    per weight. Reference: onebit_sparse_mul/__init__.py:101-145."""
+
+    def __init__(self, infeatures: int, outfeatures: int):
+        super().__init__()
+        if infeatures % 32 != 0 or outfeatures % 64 != 0:
+            raise ValueError("`infeatures` must be divisible by 32 and `outfeatures` by 64.")
+        self.infeatures = infeatures
+        self.outfeatures = outfeatures
+        self.register_buffer("packed_binary_sparse", torch.zeros((infeatures // 2, outfeatures // 8), dtype=torch.uint8))
+        self.register_buffer("meta", torch.zeros((outfeatures, infeatures // 16), dtype=torch.int16))
+        self.vaild = False
+        self._prepared = None
+
+    def pack(self, weight):
+        """weight (outfeatures, infeatures): prune to 2:4 by magnitude, keep the signs.
+        Reference: onebit_sparse_mul/__init__.py:130-145."""
+        if tuple(weight.shape) != (self.outfeatures, self.infeatures):
+            raise ValueError(f"weight must have shape ({self.outfeatures}, {self.infeatures})")
+        w = weight * mask_creator(weight).to(weight.dtype)
+        if w.dtype not in (torch.half, torch.bfloat16, torch.int32):
+            w = w.to(torch.half)
+        sparse, meta = sparse_semi_structured_from_dense_cutlass(w)
+        bits = binary_quant(sparse).T.contiguous()
+        self.packed_binary_sparse = pack_binary(bits)
+        self.meta = meta
+        self.vaild = True
+        self._prepared = None
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        super()._load_from_state_dict(*args, **kwargs)
+        self.vaild = True
+        self._prepared = None
+
+    def forward(self, x):
+        if not self.vaild:
+            raise NotImplementedError("the BinaryLinear_2_4 layer holds no packed weight: call pack() first")
+        if self._prepared is None or self._prepared.buffer.device != x.device:
+            self._prepared = PreparedWeight(self.packed_binary_sparse.to(x.device), self.meta.to(x.device))
+        lead = x.shape[:-1]
+        b = x.reshape(-1, self.infeatures).to(torch.float16).T.contiguous()  # (k, batch)
+        out = self._prepared.matmul(b, out_dtype=torch.float16)           # (outfeatures, batch)
+        return out.T.reshape(*lead, self.outfeatures).to(x.dtype)

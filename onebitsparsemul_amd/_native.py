@@ -1,0 +1,140 @@
+"""ctypes loader of libonebitmul.so (the C ABI of include/onebit_sparse_tensor.h). There is no fallback:
+if the library is missing or a call fails, an exception is raised."""
+import ctypes
+import os
+
+import torch
+
+_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_DIR, "libonebitmul.so")
+
+F32, F16 = 0, 1
+META_REFERENCE, META_CUTLASS, META_LOGICAL = 0, 1, 2
+
+EXPORTS = (
+    "onebit_sparse_matmul", "onebit_sparse_matmul_ex", "onebit_sparse_prepared_bytes", "onebit_sparse_prepare",
+    "onebit_sparse_matmul_prepared", "onebit_sparse_last_error", "onebit_sparse_set_tile_config",
+    "onebit_sparse_set_skinny_enabled",
+)
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(f"{LIB_PATH} is missing: run `python -m onebitsparsemul_amd.build` (needs hipcc)")
+        L = ctypes.CDLL(LIB_PATH)
+        vp, i32, f32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+        L.onebit_sparse_matmul.restype = None
+        L.onebit_sparse_matmul.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32]
+        L.onebit_sparse_matmul_ex.restype = i32
+        L.onebit_sparse_matmul_ex.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, i32, i32, vp]
+        L.onebit_sparse_prepared_bytes.restype = ctypes.c_size_t
+        L.onebit_sparse_prepared_bytes.argtypes = [i32, i32]
+        L.onebit_sparse_prepare.restype = i32
+        L.onebit_sparse_prepare.argtypes = [vp, vp, i32, i32, i32, vp, vp]
+        L.onebit_sparse_matmul_prepared.restype = i32
+        L.onebit_sparse_matmul_prepared.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, i32, vp]
+        L.onebit_sparse_last_error.restype = ctypes.c_char_p
+        L.onebit_sparse_last_error.argtypes = []
+        L.onebit_sparse_set_tile_config.restype = None
+        L.onebit_sparse_set_tile_config.argtypes = [i32]
+        L.onebit_sparse_set_skinny_enabled.restype = None
+        L.onebit_sparse_set_skinny_enabled.argtypes = [i32]
+        _lib = L
+    return _lib
+
+
+def last_error():
+    return lib().onebit_sparse_last_error().decode()
+
+
+def _check(rc):
+    if rc != 0:
+        raise RuntimeError(f"libonebitmul: {last_error()} (status {rc})")
+
+
+def _dtype_code(t):
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.float16:
+        return F16
+    raise TypeError(f"C / D must be float32 or float16, got {t.dtype}")
+
+
+def _stream(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _require_cuda(*tensors):
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ValueError("all operands must live on the GPU")
+        if not t.is_contiguous():
+            raise ValueError("all operands must be contiguous")
+        if dev is not None and t.device != dev:
+            raise ValueError("all operands must be on the same device")
+        dev = t.device
+    return dev
+
+
+def prepared_bytes(m, k):
+    return lib().onebit_sparse_prepared_bytes(m, k)
+
+
+def prepare(a, meta, m, k, layout=META_REFERENCE):
+    """Reorder (a bits, metadata) into the operand the kernels consume. Returns a uint8 device tensor."""
+    dev = _require_cuda(a, meta)
+    if a.numel() * a.element_size() != m * k // 16 or meta.numel() * meta.element_size() != m * k // 8:
+        raise ValueError("operand sizes do not match m, k")
+    out = torch.empty(prepared_bytes(m, k), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib().onebit_sparse_prepare(a.data_ptr(), meta.data_ptr(), m, k, layout, out.data_ptr(), _stream(a)))
+    return out
+
+
+def matmul_prepared(prepared, b, d, m, n, k, c=None, alpha=1.0, beta=0.0):
+    dev = _require_cuda(prepared, b, d, c)
+    if b.dtype != torch.float16 or tuple(b.shape) != (k, n):
+        raise ValueError("B must be float16 of shape (k, n)")
+    if tuple(d.shape) != (m, n) or (c is not None and tuple(c.shape) != (m, n)):
+        raise ValueError("C / D must have shape (m, n)")
+    if prepared.numel() != prepared_bytes(m, k):
+        raise ValueError("prepared operand does not match m, k")
+    with torch.cuda.device(dev):
+        _check(lib().onebit_sparse_matmul_prepared(
+            prepared.data_ptr(), b.data_ptr(), c.data_ptr() if c is not None else None, d.data_ptr(), m, n, k,
+            alpha, beta, _dtype_code(c) if c is not None else F32, _dtype_code(d), _stream(b)))
+    return d
+
+
+def matmul_ex(a, b, meta, d, m, n, k, c=None, alpha=1.0, beta=0.0, layout=META_REFERENCE):
+    dev = _require_cuda(a, b, meta, d, c)
+    if b.dtype != torch.float16 or tuple(b.shape) != (k, n):
+        raise ValueError("B must be float16 of shape (k, n)")
+    with torch.cuda.device(dev):
+        _check(lib().onebit_sparse_matmul_ex(
+            a.data_ptr(), b.data_ptr(), c.data_ptr() if c is not None else None, d.data_ptr(), meta.data_ptr(), m, n,
+            k, alpha, beta, _dtype_code(c) if c is not None else F32, _dtype_code(d), layout, _stream(b)))
+    return d
+
+
+def matmul_legacy(a, b, c, d, meta, m, n, k):
+    """The 8-argument entry point: fp32 C/D, alpha = 1, beta = 0, default stream."""
+    dev = _require_cuda(a, b, c, d, meta)
+    with torch.cuda.device(dev):
+        lib().onebit_sparse_matmul(a.data_ptr(), b.data_ptr(), c.data_ptr(), d.data_ptr(), meta.data_ptr(), m, n, k)
+    return d
+
+
+def set_tile_config(cfg):
+    lib().onebit_sparse_set_tile_config(cfg)
+
+
+def set_skinny_enabled(flag):
+    lib().onebit_sparse_set_skinny_enabled(1 if flag else 0)

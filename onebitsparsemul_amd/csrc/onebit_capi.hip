@@ -1,0 +1,214 @@
+// C ABI of libonebitmul (declared in include/onebit_sparse_tensor.h): argument validation, per-device
+// workspaces, kernel selection. Host code only; the kernels live in onebit_kernels.hip.
+// Counterpart of the reference's host launcher csrc/kernel_lib.cu:23-97.
+#include "onebit_sparse_tensor.h"
+#include "onebit_device.h"
+#include "onebit_launch.h"
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <mutex>
+#include <string>
+
+namespace {
+
+thread_local std::string g_last_error;
+std::atomic<int> g_tile_config{-1};
+std::atomic<int> g_skinny_enabled{1};
+
+int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
+
+#define ONEBIT_HIP(expr)                                                                         \
+  do {                                                                                           \
+    hipError_t st_ = (expr);                                                                     \
+    if (st_ != hipSuccess)                                                                       \
+      return fail(ONEBIT_ERR_HIP, "HIP error '%s' from %s", hipGetErrorString(st_), #expr);      \
+  } while (0)
+
+constexpr int kMaxDevices = 64;
+
+// Library-owned device memory: the reordered operand of the one-call entry points, the split-K partial
+// sums and the arrival counters of the skinny kernel. Grow-only, one set per device, freed at process exit
+// by the runtime. Work that uses it is ordered by the caller's stream.
+struct DeviceState {
+  std::mutex mu;
+  void* prep = nullptr;
+  size_t prep_bytes = 0;
+  float* partials = nullptr;
+  size_t partial_bytes = 0;
+  int* counters = nullptr;
+  size_t counter_count = 0;
+};
+DeviceState g_dev[kMaxDevices];
+
+int grow(void** ptr, size_t* have, size_t need, bool zero, hipStream_t stream) {
+  if (need <= *have) return ONEBIT_OK;
+  if (*ptr) {
+    // earlier work on any stream may still read the old buffer
+    ONEBIT_HIP(hipDeviceSynchronize());
+    ONEBIT_HIP(hipFree(*ptr));
+    *ptr = nullptr;
+    *have = 0;
+  }
+  const size_t bytes = (need + 4095) & ~size_t(4095);
+  ONEBIT_HIP(hipMalloc(ptr, bytes));
+  if (zero) ONEBIT_HIP(hipMemsetAsync(*ptr, 0, bytes, stream));
+  *have = bytes;
+  return ONEBIT_OK;
+}
+
+int check_shape(int m, int n, int k) {
+  if (m <= 0 || n <= 0 || k <= 0) return fail(ONEBIT_ERR_ARGUMENT, "m, n, k must be positive (got %d, %d, %d)", m, n, k);
+  if (m % 64 != 0) return fail(ONEBIT_ERR_ARGUMENT, "m = %d must be a multiple of 64 (metadata layout)", m);
+  if (k % 32 != 0) return fail(ONEBIT_ERR_ARGUMENT, "k = %d must be a multiple of 32 (metadata layout)", k);
+  return ONEBIT_OK;
+}
+
+int check_dtype(int c_dtype, int d_dtype) {
+  if ((c_dtype != ONEBIT_DTYPE_F32 && c_dtype != ONEBIT_DTYPE_F16) ||
+      (d_dtype != ONEBIT_DTYPE_F32 && d_dtype != ONEBIT_DTYPE_F16))
+    return fail(ONEBIT_ERR_ARGUMENT, "dtype codes must be 0 (fp32) or 1 (fp16), got c=%d d=%d", c_dtype, d_dtype);
+  return ONEBIT_OK;
+}
+
+int pick_tile(int m, int n) {
+  const int forced = g_tile_config.load();
+  if (forced >= 0) return forced;
+  auto tiles = [&](int bm, int bn) { return (long)((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
+  if (tiles(512, 128) >= 256) return onebit::kTile512x128;
+  if (tiles(256, 128) >= 192) return onebit::kTile256x128;
+  return onebit::kTile128x128;
+}
+
+int matmul_prepared_impl(const void* prepared, const void* b, const void* c, void* d, int m, int n, int k, float alpha,
+                         float beta, int c_dtype, int d_dtype, hipStream_t stream) {
+  if (!prepared || !b || !d) return fail(ONEBIT_ERR_ARGUMENT, "null operand pointer");
+  if (beta != 0.f && !c) return fail(ONEBIT_ERR_ARGUMENT, "c must not be null when beta != 0");
+  const int kc_total = (k + onebit::kChunkK - 1) / onebit::kChunkK;
+
+  if (n <= 32 && g_skinny_enabled.load()) {
+    int device = 0;
+    ONEBIT_HIP(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) return fail(ONEBIT_ERR_HIP, "device index %d out of range", device);
+    DeviceState& ds = g_dev[device];
+    onebit::SkinnyArgs args{};
+    args.prep = static_cast<const uint8_t*>(prepared);
+    args.b = static_cast<const _Float16*>(b);
+    args.c = c;
+    args.d = d;
+    args.m = m; args.n = n; args.k = k;
+    args.kc_total = kc_total;
+    args.alpha = alpha; args.beta = beta;
+    args.c_f16 = c_dtype == ONEBIT_DTYPE_F16;
+    args.d_f16 = d_dtype == ONEBIT_DTYPE_F16;
+    const int sk = onebit::skinny_pick_sk(m, k);
+    args.splits = (kc_total + sk - 1) / sk;
+    {
+      std::lock_guard<std::mutex> lock(ds.mu);
+      if (args.splits > 1) {
+        const int row_groups = (m + onebit::skinny_rows_per_group() - 1) / onebit::skinny_rows_per_group();
+        int rc = grow(reinterpret_cast<void**>(&ds.partials), &ds.partial_bytes,
+                      (size_t)args.splits * m * n * sizeof(float), false, stream);
+        if (rc) return rc;
+        size_t counter_bytes = ds.counter_count * sizeof(int);
+        rc = grow(reinterpret_cast<void**>(&ds.counters), &counter_bytes, (size_t)row_groups * sizeof(int), true, stream);
+        if (rc) return rc;
+        ds.counter_count = counter_bytes / sizeof(int);
+      }
+      args.partials = ds.partials;
+      args.counters = ds.counters;
+    }
+    ONEBIT_HIP(onebit::launch_skinny(args, sk, stream));
+    return ONEBIT_OK;
+  }
+
+  onebit::GemmArgs args{};
+  args.prep = static_cast<const uint8_t*>(prepared);
+  args.b = static_cast<const _Float16*>(b);
+  args.c = c;
+  args.d = d;
+  args.m = m; args.n = n; args.k = k;
+  args.kc_total = kc_total;
+  args.alpha = alpha; args.beta = beta;
+  args.c_f16 = c_dtype == ONEBIT_DTYPE_F16;
+  args.d_f16 = d_dtype == ONEBIT_DTYPE_F16;
+  ONEBIT_HIP(onebit::launch_gemm(args, pick_tile(m, n), stream));
+  return ONEBIT_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* onebit_sparse_last_error(void) { return g_last_error.c_str(); }
+
+void onebit_sparse_set_tile_config(int tile_config) { g_tile_config.store(tile_config); }
+void onebit_sparse_set_skinny_enabled(int enabled) { g_skinny_enabled.store(enabled ? 1 : 0); }
+
+size_t onebit_sparse_prepared_bytes(int m, int k) {
+  if (m <= 0 || k <= 0) return 0;
+  return onebit::prepared_bytes(m, k);
+}
+
+int onebit_sparse_prepare(const void* a, const void* e, int m, int k, int meta_layout, void* prepared, void* stream) {
+  g_last_error.clear();
+  if (int rc = check_shape(m, 1, k)) return rc;
+  if (!a || !e || !prepared) return fail(ONEBIT_ERR_ARGUMENT, "null operand pointer");
+  if (meta_layout < ONEBIT_META_REFERENCE || meta_layout > ONEBIT_META_LOGICAL)
+    return fail(ONEBIT_ERR_ARGUMENT, "unknown metadata layout %d", meta_layout);
+  ONEBIT_HIP(onebit::launch_prepare(a, e, prepared, m, k, meta_layout, static_cast<hipStream_t>(stream)));
+  return ONEBIT_OK;
+}
+
+int onebit_sparse_matmul_prepared(const void* prepared, const void* b, const void* c, void* d, int m, int n, int k,
+                                  float alpha, float beta, int c_dtype, int d_dtype, void* stream) {
+  g_last_error.clear();
+  if (int rc = check_shape(m, n, k)) return rc;
+  if (int rc = check_dtype(c_dtype, d_dtype)) return rc;
+  return matmul_prepared_impl(prepared, b, c, d, m, n, k, alpha, beta, c_dtype, d_dtype, static_cast<hipStream_t>(stream));
+}
+
+int onebit_sparse_matmul_ex(const void* a, const void* b, const void* c, void* d, const void* e, int m, int n, int k,
+                            float alpha, float beta, int c_dtype, int d_dtype, int meta_layout, void* stream) {
+  g_last_error.clear();
+  if (int rc = check_shape(m, n, k)) return rc;
+  if (int rc = check_dtype(c_dtype, d_dtype)) return rc;
+  if (!a || !b || !d || !e) return fail(ONEBIT_ERR_ARGUMENT, "null operand pointer");
+  if (beta != 0.f && !c) return fail(ONEBIT_ERR_ARGUMENT, "c must not be null when beta != 0");
+  if (meta_layout < ONEBIT_META_REFERENCE || meta_layout > ONEBIT_META_LOGICAL)
+    return fail(ONEBIT_ERR_ARGUMENT, "unknown metadata layout %d", meta_layout);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int device = 0;
+  ONEBIT_HIP(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) return fail(ONEBIT_ERR_HIP, "device index %d out of range", device);
+  DeviceState& ds = g_dev[device];
+  void* prep = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(ds.mu);
+    if (int rc = grow(&ds.prep, &ds.prep_bytes, onebit::prepared_bytes(m, k), false, s)) return rc;
+    prep = ds.prep;
+  }
+  ONEBIT_HIP(onebit::launch_prepare(a, e, prep, m, k, meta_layout, s));
+  return matmul_prepared_impl(prep, b, c, d, m, n, k, alpha, beta, c_dtype, d_dtype, s);
+}
+
+void onebit_sparse_matmul(void* a, void* b, void* c, void* d, void* e, int m, int n, int k) {
+  const int rc = onebit_sparse_matmul_ex(a, b, c, d, e, m, n, k, 1.0f, 0.0f, ONEBIT_DTYPE_F32, ONEBIT_DTYPE_F32,
+                                         ONEBIT_META_REFERENCE, nullptr);
+  if (rc != ONEBIT_OK) {
+    fprintf(stderr, "Got onebit_sparse_matmul error: %s\n", g_last_error.c_str());
+    exit(EXIT_FAILURE);
+  }
+}
+
+}  // extern "C"

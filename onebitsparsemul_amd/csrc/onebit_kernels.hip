@@ -1,0 +1,573 @@
+// gfx950 kernels of the one-bit 2:4 sparse GEMM  D = alpha * A * B + beta * C.
+//   prepare_kernel  : reference operands (1-bit values, reordered 2-bit-index metadata) -> prepared operand
+//   gemm_kernel     : main SMFMAC kernel (B staged through LDS, A expanded in registers)
+//   skinny_kernel   : split-K kernel for N <= 32 (decode shapes)
+// Replaces the CUTLASS specialisations of the reference (csrc/kernel.h:13-72, csrc/threadblock.h:62-233,
+// csrc/warp.h:18-690) with code written for 64-wide wavefronts; nothing is translated from them.
+#include "onebit_device.h"
+#include "onebit_launch.h"
+#include <type_traits>
+
+namespace onebit {
+
+// =====================================================================================================
+// prepare_kernel: one wavefront per prepared block (rb, kc).
+// Reads  a : bit (r, j) of the (m x k/2) column-major one-bit matrix = bit (r + j m) % 8 of byte (r + j m) / 8
+//            (csrc/kernel_lib.cu:28,37; produced by onebit_sparse_mul/__init__.py:139-143), 1 = +1, 0 = -1
+//        e : int16 metadata (m x k/16) in the reference's reordered layout or the CUTLASS one
+//            (_semi_structured_conversions.py:21-48,173-177)
+// Writes the block described in onebit_device.h. K is padded up to a multiple of 256 with +1 values on
+// positions 0,1 of each group; the GEMM kernels multiply that padding by zero rows of B.
+// =====================================================================================================
+__global__ __launch_bounds__(64) void prepare_kernel(const uint8_t* __restrict__ a, const uint16_t* __restrict__ e,
+                                                     uint8_t* __restrict__ prep, int m, int k, int kc_total,
+                                                     int layout) {
+  const int kc = blockIdx.x, rb = blockIdx.y, lane = threadIdx.x;
+  const int i = lane & 31, ga = lane >> 5;
+  const int64_t r = (int64_t)rb * kRowBlock + i;
+  const int ncols = k / 16;
+  uint32_t meta[4] = {0, 0, 0, 0};
+  uint32_t sign[2] = {0, 0};
+  if (r < m) {
+#pragma unroll
+    for (int s = 0; s < kStepsPerChunk; ++s) {
+      const int c = kc * 16 + 2 * s + ga;
+      uint32_t mv = 0x4444u;
+      uint32_t neg = 0;  // bit t set: kept value t of this step is -1
+      if (c < ncols) {
+        int64_t off;
+        if (layout == 0) off = meta_offset_reference(r, c, m);
+        else if (layout == 1) off = meta_offset_cutlass(r, c, m);
+        else off = r * ncols + c;
+        mv = e[off];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          const int64_t pos = r + (int64_t)(8 * c + t) * m;
+          const uint32_t bit = (a[pos >> 3] >> (pos & 7)) & 1u;
+          neg |= (bit ^ 1u) << t;
+        }
+      }
+      meta[s >> 1] |= mv << (16 * (s & 1));
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const int j = 4 * (s & 3) + p;
+        sign[s >> 2] |= ((neg >> (2 * p)) & 1u) << (15 - j);
+        sign[s >> 2] |= ((neg >> (2 * p + 1)) & 1u) << (31 - j);
+      }
+    }
+  } else {
+    meta[0] = meta[1] = meta[2] = meta[3] = 0x44444444u;
+  }
+  uint8_t* block = prep + ((size_t)rb * kc_total + kc) * kBlockBytes;
+  u32x4_t mvec = {meta[0], meta[1], meta[2], meta[3]};
+  u32x2_t svec = {sign[0], sign[1]};
+  *reinterpret_cast<u32x4_t*>(block + lane * 16) = mvec;
+  *reinterpret_cast<u32x2_t*>(block + kSignOffset + lane * 8) = svec;
+}
+
+// =====================================================================================================
+// Main kernel.
+// Workgroup = 4 wavefronts arranged WM x WN; each wavefront owns FM x FN accumulator tiles of 32 x 32.
+// B is staged through LDS in stages of 64 K rows; the LDS image of a stage is row-major (N contiguous)
+// with the 16-byte column chunks of row r XOR-swizzled so that the four rows a 16-lane group touches in
+// one transpose read fall into different bank groups.
+// =====================================================================================================
+constexpr int kStageK = 64;
+constexpr int kStages = 4;  // LDS ring; one prepared-operand chunk (256 K) = one trip around the ring
+
+template <int BN>
+__device__ __forceinline__ int chunk_swizzle(int row) {
+  // 16-byte chunk index XOR; rows r..r+3 must land in four different 64-byte bank groups.
+  return (BN >= 128) ? ((row & 3) << 2) : (((row >> 1) & 1) << 2);
+}
+
+template <int WM, int WN, int FM, int FN>
+struct TileShape {
+  static constexpr int BM = WM * FM * 32;
+  static constexpr int BN = WN * FN * 32;
+  static constexpr int CH = BN / 8;                       // 16-byte chunks per LDS row
+  static constexpr int NL = kStageK * CH / 256;           // chunk copies per thread per stage
+  static constexpr int STAGE_BYTES = kStageK * BN * 2;
+  static constexpr int LDS_B_BYTES = kStages * STAGE_BYTES;
+  static constexpr int NA = ((BM / 32) * 1536 + 4095) / 4096;  // 1 KiB A copies per wavefront per K chunk
+  static constexpr int LDS_BYTES = LDS_B_BYTES + NA * 4096;
+  static_assert(WM * WN == 4, "four wavefronts per workgroup");
+  static_assert(NL >= 1, "tile too narrow for the copy pattern");
+};
+
+// XCD-aware tile order: workgroup b runs on XCD b % 8, so XCD x is given a contiguous range of the tile
+// list, and the list itself walks tiles in groups of eight row tiles so that the ~32 tiles resident on
+// one XCD share A row panels and B column panels in that XCD's L2.
+__device__ __forceinline__ void tile_of_block(int b, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  const int per = total / 8, rem = total % 8;
+  const int x = b % 8, local = b / 8;
+  const int v = x * per + (x < rem ? x : rem) + local;
+  constexpr int GROUP_M = 8;
+  const int in_group = GROUP_M * tiles_n;
+  const int g = v / in_group;
+  const int first_m = g * GROUP_M;
+  const int gsz = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+  const int w = v % in_group;
+  tm = first_m + w % gsz;
+  tn = w / gsz;
+}
+
+// One stage (64 K = two SMFMAC K steps) of a wavefront's FM x FN tile.
+template <int FM, int FN, int BN, int STAGE_IN_CHUNK>
+__device__ __forceinline__ void compute_stage(const char* stage_lds, const AChunk (&a)[FM], float16_t (&acc)[FM][FN],
+                                              const int (&frag_off)[FN], int lane_row_off) {
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    constexpr int dummy = 0;
+    (void)dummy;
+    half16_t bv[FN];
+#pragma unroll
+    for (int fn = 0; fn < FN; ++fn) {
+      u32x8_t raw;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row_const = ks * 32 + 4 * (q & 1) + 16 * (q >> 1);
+        const u32x2_t t = lds_read_tr16(stage_lds + lane_row_off + row_const * (BN * 2) + frag_off[fn]);
+        raw[2 * q] = t.x;
+        raw[2 * q + 1] = t.y;
+      }
+      bv[fn] = __builtin_bit_cast(half16_t, raw);
+    }
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm) {
+      half8_t av;
+      if (ks == 0) av = expand_signs<2 * STAGE_IN_CHUNK>(a[fm]);
+      else av = expand_signs<2 * STAGE_IN_CHUNK + 1>(a[fm]);
+#pragma unroll
+      for (int fn = 0; fn < FN; ++fn) {
+        if (ks == 0) acc[fm][fn] = smfmac_step<2 * STAGE_IN_CHUNK>(a[fm], av, bv[fn], acc[fm][fn]);
+        else acc[fm][fn] = smfmac_step<2 * STAGE_IN_CHUNK + 1>(a[fm], av, bv[fn], acc[fm][fn]);
+      }
+    }
+  }
+}
+
+template <int WM, int WN, int FM, int FN, bool DMA>
+__global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
+  using TS = TileShape<WM, WN, FM, FN>;
+  constexpr int BM = TS::BM, BN = TS::BN, CH = TS::CH, NL = TS::NL;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in a scalar register
+  const int wm = wave / WN, wn = wave % WN;
+  int tile_m, tile_n;
+  tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  const int row0 = tile_m * BM + wm * FM * 32;  // first row of this wavefront
+  const int n0 = tile_n * BN;                   // first column of the workgroup
+  const int col0 = n0 + wn * FN * 32;           // first column of this wavefront
+
+  // ---- A operand addressing (prepared blocks) ----
+  const int rb_total = p.m / kRowBlock;
+  const uint8_t* a_block[FM];
+#pragma unroll
+  for (int fm = 0; fm < FM; ++fm) {
+    int rb = row0 / kRowBlock + fm;
+    if (rb >= rb_total) rb = rb_total - 1;  // rows past M: compute on valid data, never stored
+    a_block[fm] = p.prep + (size_t)rb * p.kc_total * kBlockBytes;
+  }
+
+  // ---- B fragment addressing inside a stage ----
+  const int i16 = lane & 15;
+  const int gb = lane >> 5;
+  const int c8 = ((lane & 31) >> 4) * 4 + (i16 & 3);  // 8-byte chunk inside the 32-column fragment
+  const int lane_row = 8 * gb + (i16 >> 2);           // + compile-time row constants
+  const int lane_row_off = lane_row * (BN * 2);
+  int frag_off[FN];
+#pragma unroll
+  for (int fn = 0; fn < FN; ++fn) {
+    const int lc = 4 * (wn * FN + fn) + (c8 >> 1);
+    frag_off[fn] = ((lc ^ chunk_swizzle<BN>(lane_row)) << 4) + (c8 & 1) * 8;
+  }
+
+  float16_t acc[FM][FN];
+#pragma unroll
+  for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+    for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[fm][fn][v] = 0.f;
+
+  const int stages_total = (p.k + kStageK - 1) / kStageK;
+  const int chunks = (stages_total + kStages - 1) / kStages;
+
+  if constexpr (DMA) {
+    // ---- asynchronous copy pattern for B: NL chunk copies per thread per stage ----
+    // copy i of wavefront w fills LDS slots [(4 i + w) * 64, +64) of the stage; slot s = (row, physical chunk).
+    const char* gsrc[NL];
+    uint32_t lds_dst[NL];
+    const uint32_t smem_base = lds_offset_of(smem);
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int slot = (4 * i + wave) * 64 + lane;
+      const int row = slot / CH, pc = slot % CH;
+      const int lc = pc ^ chunk_swizzle<BN>(row);
+      int col = n0 + 8 * lc;
+      if (col >= p.n) col = n0;  // columns past N: any valid address will do, the results are not stored
+      gsrc[i] = reinterpret_cast<const char*>(p.b) + ((size_t)row * p.n + col) * 2;
+      lds_dst[i] = smem_base + (4 * i + wave) * 1024;
+    }
+    const size_t stage_stride = (size_t)kStageK * p.n * 2;
+    int next_stage = 0;  // next stage index to copy
+    auto issue_b = [&](int ring) {
+#pragma unroll
+      for (int i = 0; i < NL; ++i) lds_dma16(gsrc[i], lds_dst[i] + ring * TS::STAGE_BYTES);
+      // past the last stage the same (valid) rows are copied again so that the number of copies in
+      // flight, which the vmcnt waits below rely on, stays constant
+      if (next_stage + 1 < stages_total) {
+#pragma unroll
+        for (int i = 0; i < NL; ++i) gsrc[i] += stage_stride;
+      }
+      ++next_stage;
+    };
+
+    // ---- asynchronous copy pattern for A: the workgroup's BM/32 prepared blocks of one K chunk ----
+    // LDS image = the blocks back to back; NA copies of 1 KiB per wavefront (the tail past the last block
+    // re-copies the first block into padding so that every wavefront issues the same number of requests).
+    constexpr int NA = TS::NA;
+    char* a_lds = smem + TS::LDS_B_BYTES;
+    const char* a_src[NA];
+    uint32_t a_dst[NA];
+    {
+      const int rb0 = tile_m * (BM / kRowBlock);
+#pragma unroll
+      for (int j = 0; j < NA; ++j) {
+        const int byte = (4 * j + wave) * 1024 + lane * 16;
+        int blk = byte / kBlockBytes, off = byte % kBlockBytes;
+        if (blk >= BM / kRowBlock) blk = 0;
+        int rb = rb0 + blk;
+        if (rb >= rb_total) rb = rb_total - 1;
+        a_src[j] = reinterpret_cast<const char*>(p.prep) + (size_t)rb * p.kc_total * kBlockBytes + off;
+        a_dst[j] = smem_base + TS::LDS_B_BYTES + (4 * j + wave) * 1024;
+      }
+    }
+    int next_chunk = 0;
+    auto issue_a = [&]() {
+#pragma unroll
+      for (int j = 0; j < NA; ++j) lds_dma16(a_src[j], a_dst[j]);
+      if (next_chunk + 1 < chunks) {
+#pragma unroll
+        for (int j = 0; j < NA; ++j) a_src[j] += kBlockBytes;
+      }
+      ++next_chunk;
+    };
+    const char* a_frag_lds[FM];
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm) a_frag_lds[fm] = a_lds + (wm * FM + fm) * kBlockBytes;
+
+    // Request order: A(0) B(0) B(1) B(2) | per chunk c: s0: B(4c+3)  s1: B(4c+4) A(c+1)  s2: B(4c+5)  s3: B(4c+6)
+    issue_a();
+#pragma unroll
+    for (int s = 0; s < kStages - 1; ++s) issue_b(s);
+
+    for (int kc = 0; kc < chunks; ++kc) {
+      AChunk a_cur[FM];
+      // stage 0: needs B(4c) and A(c); newer requests: two B stages
+      wait_vmcnt<2 * NL>();
+      __builtin_amdgcn_s_barrier();
+      issue_b(3);
+#pragma unroll
+      for (int fm = 0; fm < FM; ++fm) a_cur[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);
+      compute_stage<FM, FN, BN, 0>(smem + 0 * TS::STAGE_BYTES, a_cur, acc, frag_off, lane_row_off);
+
+      // stage 1: newer requests: two B stages. All wavefronts have read A(c) before this barrier.
+      wait_vmcnt<2 * NL>();
+      __builtin_amdgcn_s_barrier();
+      issue_b(0);
+      issue_a();
+      if (kc * kStages + 1 < stages_total)
+        compute_stage<FM, FN, BN, 1>(smem + 1 * TS::STAGE_BYTES, a_cur, acc, frag_off, lane_row_off);
+
+      // stage 2: newer requests: two B stages and one A chunk
+      wait_vmcnt<2 * NL + NA>();
+      __builtin_amdgcn_s_barrier();
+      issue_b(1);
+      if (kc * kStages + 2 < stages_total)
+        compute_stage<FM, FN, BN, 2>(smem + 2 * TS::STAGE_BYTES, a_cur, acc, frag_off, lane_row_off);
+
+      wait_vmcnt<2 * NL + NA>();
+      __builtin_amdgcn_s_barrier();
+      issue_b(2);
+      if (kc * kStages + 3 < stages_total)
+        compute_stage<FM, FN, BN, 3>(smem + 3 * TS::STAGE_BYTES, a_cur, acc, frag_off, lane_row_off);
+    }
+    wait_vmcnt<0>();  // drain the copies issued past the end before the LDS is released
+  } else {
+    // ---- generic path: any N, any K % 32 == 0, any alignment. One stage at a time, element copies. ----
+    for (int kc = 0; kc < chunks; ++kc) {
+      AChunk a_cur[FM];
+#pragma unroll
+      for (int fm = 0; fm < FM; ++fm) a_cur[fm] = load_a_chunk(a_block[fm] + (size_t)kc * kBlockBytes, lane);
+      auto fill = [&](int stage) {
+        const int k0 = (kc * kStages + stage) * kStageK;
+        __syncthreads();
+        for (int idx = tid; idx < kStageK * BN; idx += 256) {
+          const int row = idx / BN, col = idx % BN;
+          _Float16 v = (_Float16)0.f;
+          if (k0 + row < p.k && n0 + col < p.n) v = p.b[(size_t)(k0 + row) * p.n + n0 + col];
+          const int lc = (col >> 3) ^ chunk_swizzle<BN>(row);
+          *reinterpret_cast<_Float16*>(smem + row * (BN * 2) + (lc << 4) + (col & 7) * 2) = v;
+        }
+        __syncthreads();
+      };
+      if (kc * kStages + 0 < stages_total) { fill(0); compute_stage<FM, FN, BN, 0>(smem, a_cur, acc, frag_off, lane_row_off); }
+      if (kc * kStages + 1 < stages_total) { fill(1); compute_stage<FM, FN, BN, 1>(smem, a_cur, acc, frag_off, lane_row_off); }
+      if (kc * kStages + 2 < stages_total) { fill(2); compute_stage<FM, FN, BN, 2>(smem, a_cur, acc, frag_off, lane_row_off); }
+      if (kc * kStages + 3 < stages_total) { fill(3); compute_stage<FM, FN, BN, 3>(smem, a_cur, acc, frag_off, lane_row_off); }
+    }
+  }
+
+  // ---- epilogue: D = alpha * acc + beta * C (csrc/kernel.h:27-31), fp16 (RNE) or fp32 output ----
+  const int col_lane = lane & 31;
+  const int row_lane = 4 * (lane >> 5);
+#pragma unroll
+  for (int fm = 0; fm < FM; ++fm) {
+#pragma unroll
+    for (int fn = 0; fn < FN; ++fn) {
+      const int col = col0 + fn * 32 + col_lane;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = row0 + fm * 32 + 8 * (v / 4) + row_lane + (v % 4);
+        if (row < p.m && col < p.n) {
+          const size_t o = (size_t)row * p.n + col;
+          float x = p.alpha * acc[fm][fn][v];
+          if (p.beta != 0.f) {
+            const float cv = p.c_f16 ? (float)reinterpret_cast<const _Float16*>(p.c)[o]
+                                     : reinterpret_cast<const float*>(p.c)[o];
+            x = x + p.beta * cv;
+          }
+          if (p.d_f16) reinterpret_cast<_Float16*>(p.d)[o] = (_Float16)x;
+          else reinterpret_cast<float*>(p.d)[o] = x;
+        }
+      }
+    }
+  }
+}
+
+// =====================================================================================================
+// skinny_kernel: N <= 32 (decode shapes). HBM-bound: every byte of the prepared operand is read once.
+// Workgroup = 4 wavefronts sharing one K slice (SK chunks of 256) of B, staged into LDS as a zero-padded
+// [k][NC]-image; wavefront w owns R row blocks (32 rows each). grid = (row groups, K splits).
+// With more than one K split, partial sums go to a workspace and the last workgroup to finish a row group
+// adds them in split order (deterministic) and applies the epilogue.
+// =====================================================================================================
+template <int R, int SK, int NC>
+__global__ __launch_bounds__(256) void skinny_kernel(SkinnyArgs p) {
+  constexpr int RS = NC * 2;  // bytes per LDS row
+  __shared__ __attribute__((aligned(16))) char bs[SK * kChunkK * RS];
+  __shared__ int last_flag;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int rg = blockIdx.x, split = blockIdx.y;
+  const int kc0 = split * SK;
+  const int rb_total = p.m / kRowBlock;
+  const int rb_first = (rg * 4 + wave) * R;
+
+  // weight stream first: all requests of this wavefront are in flight while B is staged
+  AChunk a[SK][R];
+#pragma unroll
+  for (int c = 0; c < SK; ++c) {
+    int kc = kc0 + c;
+    if (kc >= p.kc_total) kc = p.kc_total - 1;  // valid address; its B rows are zero
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      int rb = rb_first + r;
+      if (rb >= rb_total) rb = rb_total - 1;
+      a[c][r] = load_a_chunk(p.prep + ((size_t)rb * p.kc_total + kc) * kBlockBytes, lane);
+    }
+  }
+
+  // stage B rows [kc0*256, +SK*256) x NC columns, zero outside the matrix
+  {
+    const int k_base = kc0 * kChunkK;
+    if (NC == 16 && p.n == 16 && (reinterpret_cast<uintptr_t>(p.b) & 15) == 0) {
+      const u32x4_t* src = reinterpret_cast<const u32x4_t*>(p.b + (size_t)k_base * 16);
+      for (int idx = tid; idx < SK * kChunkK * 2; idx += 256) {
+        const int row = idx >> 1;
+        u32x4_t v = {0, 0, 0, 0};
+        if (k_base + row < p.k) v = src[idx];
+        *reinterpret_cast<u32x4_t*>(bs + idx * 16) = v;
+      }
+    } else {
+      for (int idx = tid; idx < SK * kChunkK * NC; idx += 256) {
+        const int row = idx / NC, col = idx % NC;
+        _Float16 v = (_Float16)0.f;
+        if (k_base + row < p.k && col < p.n) v = p.b[(size_t)(k_base + row) * p.n + col];
+        *reinterpret_cast<_Float16*>(bs + row * RS + col * 2) = v;
+      }
+    }
+  }
+  __syncthreads();
+
+  float16_t acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[r][v] = 0.f;
+
+  const int i16 = lane & 15, gb = lane >> 5;
+  const int half32 = (NC == 32) ? ((lane & 31) >> 4) : 0;  // NC == 16: lanes 16-31 duplicate columns 0-15
+  const char* lane_ptr = bs + (8 * gb + (i16 >> 2)) * RS + ((i16 & 3) + 4 * half32) * 8;
+
+#pragma unroll
+  for (int c = 0; c < SK; ++c) {
+    auto step = [&](auto step_tag) {
+      constexpr int STEP = decltype(step_tag)::value;
+      u32x8_t raw;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row_const = c * kChunkK + STEP * 32 + 4 * (q & 1) + 16 * (q >> 1);
+        const u32x2_t t = lds_read_tr16(lane_ptr + row_const * RS);
+        raw[2 * q] = t.x;
+        raw[2 * q + 1] = t.y;
+      }
+      const half16_t bv = __builtin_bit_cast(half16_t, raw);
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[r] = smfmac_step<STEP>(a[c][r], expand_signs<STEP>(a[c][r]), bv, acc[r]);
+    };
+    step(std::integral_constant<int, 0>{});
+    step(std::integral_constant<int, 1>{});
+    step(std::integral_constant<int, 2>{});
+    step(std::integral_constant<int, 3>{});
+    step(std::integral_constant<int, 4>{});
+    step(std::integral_constant<int, 5>{});
+    step(std::integral_constant<int, 6>{});
+    step(std::integral_constant<int, 7>{});
+  }
+
+  const int col = lane & 31;
+  const int row_lane = 4 * (lane >> 5);
+  const bool col_ok = col < p.n && (NC == 32 || (lane & 31) < 16);
+  auto store_out = [&](size_t o, float sum) {
+    float x = p.alpha * sum;
+    if (p.beta != 0.f) {
+      const float cv = p.c_f16 ? (float)reinterpret_cast<const _Float16*>(p.c)[o] : reinterpret_cast<const float*>(p.c)[o];
+      x = x + p.beta * cv;
+    }
+    if (p.d_f16) reinterpret_cast<_Float16*>(p.d)[o] = (_Float16)x;
+    else reinterpret_cast<float*>(p.d)[o] = x;
+  };
+
+  if (p.splits == 1) {
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = (rb_first + r) * kRowBlock + 8 * (v / 4) + row_lane + (v % 4);
+        if (col_ok && row < p.m) store_out((size_t)row * p.n + col, acc[r][v]);
+      }
+    return;
+  }
+
+  // ---- split-K: publish the partial tile, the last workgroup of the row group reduces ----
+  float* part = p.partials + (size_t)split * p.m * p.n;
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = (rb_first + r) * kRowBlock + 8 * (v / 4) + row_lane + (v % 4);
+      if (col_ok && row < p.m) part[(size_t)row * p.n + col] = acc[r][v];
+    }
+  __threadfence();  // make the partial tile visible device-wide before the arrival count
+  __syncthreads();
+  if (tid == 0) {
+    const int prev = __hip_atomic_fetch_add(&p.counters[rg], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    last_flag = (prev == p.splits - 1);
+  }
+  __syncthreads();
+  if (!last_flag) return;
+  __threadfence();
+  const int rows_per_group = 4 * R * kRowBlock;
+  const int row_begin = rg * rows_per_group;
+  const int row_end = (row_begin + rows_per_group < p.m) ? row_begin + rows_per_group : p.m;
+  const int count = (row_end - row_begin) * p.n;
+  const size_t base = (size_t)row_begin * p.n;
+  const size_t split_stride = (size_t)p.m * p.n;
+  for (int idx = tid; idx < count; idx += 256) {
+    float sum = 0.f;
+    for (int s = 0; s < p.splits; ++s) sum += __builtin_nontemporal_load(p.partials + s * split_stride + base + idx);
+    store_out(base + idx, sum);
+  }
+  if (tid == 0) __hip_atomic_store(&p.counters[rg], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next call
+}
+
+// =====================================================================================================
+// Host-side launchers
+// =====================================================================================================
+hipError_t launch_prepare(const void* a, const void* e, void* prep, int m, int k, int layout, hipStream_t stream) {
+  const int kc_total = (k + kChunkK - 1) / kChunkK;
+  const int rb_total = (m + kRowBlock - 1) / kRowBlock;
+  dim3 grid(kc_total, rb_total);
+  hipLaunchKernelGGL(prepare_kernel, grid, dim3(64), 0, stream, (const uint8_t*)a, (const uint16_t*)e, (uint8_t*)prep,
+                     m, k, kc_total, layout);
+  return hipGetLastError();
+}
+
+template <int WM, int WN, int FM, int FN, bool DMA>
+static hipError_t launch_gemm_cfg(GemmArgs args, hipStream_t stream) {
+  using TS = TileShape<WM, WN, FM, FN>;
+  args.tiles_m = (args.m + TS::BM - 1) / TS::BM;
+  args.tiles_n = (args.n + TS::BN - 1) / TS::BN;
+  const int lds = DMA ? TS::LDS_BYTES : TS::STAGE_BYTES;
+  auto kern = gemm_kernel<WM, WN, FM, FN, DMA>;
+  static bool attr_done = false;  // per instantiation; racing writers store the same value
+  if (!attr_done) {
+    hipError_t st = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (st != hipSuccess) return st;
+    attr_done = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n), dim3(256), lds, stream, args);
+  return hipGetLastError();
+}
+
+hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
+  const bool aligned = (args.n % 8 == 0) && (args.k % kStageK == 0) && ((reinterpret_cast<uintptr_t>(args.b) & 15) == 0);
+  if (!aligned) return launch_gemm_cfg<4, 1, 1, 4, false>(args, stream);
+  switch (tile_config) {
+    case kTile512x128: return launch_gemm_cfg<4, 1, 4, 4, true>(args, stream);
+    case kTile256x128: return launch_gemm_cfg<4, 1, 2, 4, true>(args, stream);
+    case kTile128x128: return launch_gemm_cfg<4, 1, 1, 4, true>(args, stream);
+    case kTile256x256: return launch_gemm_cfg<2, 2, 4, 4, true>(args, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+template <int R, int SK, int NC>
+static hipError_t launch_skinny_cfg(const SkinnyArgs& args, hipStream_t stream) {
+  const int row_groups = (args.m + 4 * R * kRowBlock - 1) / (4 * R * kRowBlock);
+  hipLaunchKernelGGL((skinny_kernel<R, SK, NC>), dim3(row_groups, args.splits), dim3(256), 0, stream, args);
+  return hipGetLastError();
+}
+
+int skinny_rows_per_group() { return 4 * 2 * kRowBlock; }
+
+int skinny_pick_sk(int m, int k) {
+  const int row_groups = (m + skinny_rows_per_group() - 1) / skinny_rows_per_group();
+  const int kc_total = (k + kChunkK - 1) / kChunkK;
+  const int cand[4] = {8, 4, 2, 1};
+  for (int i = 0; i < 4; ++i) {
+    const int sk = cand[i];
+    if (row_groups * ((kc_total + sk - 1) / sk) >= 256) return sk;
+  }
+  return 1;
+}
+
+hipError_t launch_skinny(SkinnyArgs args, int sk, hipStream_t stream) {
+  const bool wide = args.n > 16;
+  switch (sk) {
+    case 1: return wide ? launch_skinny_cfg<2, 1, 32>(args, stream) : launch_skinny_cfg<2, 1, 16>(args, stream);
+    case 2: return wide ? launch_skinny_cfg<2, 2, 32>(args, stream) : launch_skinny_cfg<2, 2, 16>(args, stream);
+    case 4: return wide ? launch_skinny_cfg<2, 4, 32>(args, stream) : launch_skinny_cfg<2, 4, 16>(args, stream);
+    case 8: return wide ? launch_skinny_cfg<2, 8, 32>(args, stream) : launch_skinny_cfg<2, 8, 16>(args, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace onebit
