@@ -1,0 +1,171 @@
+"""Benchmark of the one-bit 2:4 sparse GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload square:8192]
+
+A step is one product D = A*B (prepared weight, fp16 B resident in HBM, fp32 accumulate, fp16 D). The default
+workload is the square 8192^3 problem the headline metric is quoted on; the dense-equivalent FLOP count is
+2*M*N*K (the reference's own convention, tests/kernel_test.cu:207-215). The JSON line also carries the
+roofline figures of the dominant kernel, the HBM figure of the N=16 decode shape and the CPU baseline.
+Other workloads: square:<size>, decode:<m>x<k>x<n>, prefill (4096x2048x4096, alpha=0.5, beta=1).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+CU_COUNT = 256
+CLOCK_HZ = 2.4e9
+DENSE_F16_PEAK_TFLOPS = CU_COUNT * CLOCK_HZ * 4096 / 1e12        # 2516.6: published dense fp16 MFMA peak
+SMFMAC_PEAK_TFLOPS = 2 * DENSE_F16_PEAK_TFLOPS                   # dense-equivalent rate of v_smfmac f16
+HBM_PEAK_GBS = 8000.0
+
+
+def parse_workload(text):
+    if text.startswith("square:"):
+        s = int(text.split(":")[1])
+        return dict(name=text, m=s, n=s, k=s, alpha=1.0, beta=0.0)
+    if text.startswith("decode:"):
+        m, k, n = (int(v) for v in text.split(":")[1].split("x"))
+        return dict(name=text, m=m, n=n, k=k, alpha=1.0, beta=0.0)
+    if text == "prefill":
+        return dict(name=text, m=4096, n=2048, k=4096, alpha=0.5, beta=1.0)
+    raise SystemExit(f"unknown workload {text!r}")
+
+
+def algorithmic_bytes(m, n, k, beta):
+    # a bits + metadata (= prepared operand, 1.5 bit per weight) + B + D (+ C), each counted once
+    return m * k // 16 + m * k // 8 + 2 * k * n + 2 * m * n + (2 * m * n if beta != 0.0 else 0)
+
+
+def time_launches(fn, steps, warmup):
+    """Average duration of one launch: HIP events on the stream the kernels run on (torch's current stream)."""
+    import torch
+    for _ in range(warmup):
+        fn(0)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(steps):
+        fn(i)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return start.elapsed_time(stop) / steps * 1e-3, wall / steps
+
+
+def run_gemm(w, steps, warmup):
+    import torch
+    from onebitsparsemul_amd import _native, synthetic
+    m, n, k = w["m"], w["n"], w["k"]
+    a, meta = synthetic.make_weight(m, k, seed=0x0B5A0000, device="cuda")
+    b = synthetic.make_b(k, n, seed=1, kind="normal", device="cuda")
+    c = synthetic.make_c(m, n, seed=2, device="cuda") if w["beta"] != 0.0 else None
+    prep = _native.prepare(a, meta, m, k)
+    d = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    fn = lambda i: _native.matmul_prepared(prep, b, d, m, n, k, c=c, alpha=w["alpha"], beta=w["beta"])
+    kernel_s, wall_s = time_launches(fn, steps, warmup)
+    return kernel_s, wall_s, (a, meta, b, d)
+
+
+def run_decode_rotating(m, k, n, launches=2000, copies=None):
+    """HBM-bound decode shape: rotate over enough distinct prepared weights (> 256 MiB in total, more than the
+    last-level cache) that every launch streams its weight from HBM; also time the same-buffer case."""
+    import torch
+    from onebitsparsemul_amd import _native, synthetic
+    a, meta = synthetic.make_weight(m, k, seed=3, device="cuda")
+    prep0 = _native.prepare(a, meta, m, k)
+    if copies is None:
+        copies = max(64, (768 << 20) // prep0.numel() + 1)
+    preps = [prep0] + [prep0.clone() for _ in range(copies - 1)]
+    b = synthetic.make_b(k, n, seed=4, kind="normal", device="cuda")
+    d = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    rot = lambda i: _native.matmul_prepared(preps[i % copies], b, d, m, n, k)
+    same = lambda i: _native.matmul_prepared(prep0, b, d, m, n, k)
+    t_rot, _ = time_launches(rot, launches, 50)
+    t_same, _ = time_launches(same, launches, 50)
+    nbytes = algorithmic_bytes(m, n, k, 0.0)
+    return dict(shape=f"{m}x{k}x{n}", bytes=nbytes, copies=copies, launches=launches,
+                us_per_launch_hbm=t_rot * 1e6, gbps_hbm=nbytes / t_rot / 1e9,
+                us_per_launch_cache_resident=t_same * 1e6, gbps_cache_resident=nbytes / t_same / 1e9,
+                frac_of_hbm_peak=nbytes / t_rot / 1e9 / HBM_PEAK_GBS)
+
+
+def cpu_baseline(w, operands, budget_s=15.0):
+    """oracle (kind 'port'): decompress + dense fp32 torch.matmul on the host cores, on a row slab sized for
+    about budget_s seconds; rate in the metric's unit (dense-equivalent TFLOP/s)."""
+    import torch
+    import oracle
+    a, meta, b, d = operands
+    m, n, k = w["m"], w["n"], w["k"]
+    a_h, e_h, b_h = a.cpu().numpy(), meta.cpu().numpy(), b.cpu().numpy()
+    probe_rows = min(m, 256)
+    t_probe, _, _ = oracle.cpu_baseline_gemm(a_h, b_h, e_h, m, n, k, 0, probe_rows)
+    rate = 2.0 * probe_rows * n * k / max(t_probe, 1e-9)
+    rows = int(min(m, max(probe_rows, (budget_s * rate / (2.0 * n * k)) // 64 * 64)))
+    t_mm, t_dec, out = oracle.cpu_baseline_gemm(a_h, b_h, e_h, m, n, k, 0, rows)
+    # the slab doubles as a parity spot check of the timed GPU result
+    got = d[:rows].float().cpu().numpy()
+    scale = float(abs(out).max())
+    rel = float(abs(got - w["alpha"] * out).max() / scale) if w["beta"] == 0.0 else None
+    return dict(value=2.0 * rows * n * k / t_mm / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"rows 0..{rows} of {m} (all of K={k}, N={n}): decompress {t_dec:.2f}s + fp32 torch.matmul {t_mm:.2f}s",
+                gpu_vs_oracle_rel_err_on_sample=rel)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="square:8192")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-decode", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
+    import torch
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU")
+    torch.cuda.set_device(0)
+    w = parse_workload(args.workload)
+    m, n, k = w["m"], w["n"], w["k"]
+
+    if w["name"].startswith("decode:"):
+        dec = run_decode_rotating(m, k, n, launches=max(args.steps, 200))
+        line = dict(metric="hbm_gbps_decode", value=dec["gbps_hbm"], unit="GB/s", n_gpus=1, steps=dec["launches"],
+                    warmup=50, ms_per_step=dec["us_per_launch_hbm"] * 1e-3, higher_is_better=True, scaling="weak",
+                    vs_baseline=None, dtype="f16", data="synthetic", config=dict(workload=w["name"]),
+                    roofline=dict(bound="hbm", achieved=dec["gbps_hbm"], peak=HBM_PEAK_GBS, unit="GB/s",
+                                  frac=dec["frac_of_hbm_peak"], traffic=None), decode=dec)
+        print(json.dumps(line))
+        return
+
+    kernel_s, wall_s, operands = run_gemm(w, args.steps, args.warmup)
+    tflops = 2.0 * m * n * k / kernel_s / 1e12
+    line = dict(
+        metric="dense_equiv_tflops", value=tflops, unit="TFLOP/s", n_gpus=1, steps=args.steps, warmup=args.warmup,
+        ms_per_step=kernel_s * 1e3, higher_is_better=True, scaling="weak", vs_baseline=None, dtype="f16",
+        data="synthetic",
+        config=dict(workload=w["name"], m=m, n=n, k=k, alpha=w["alpha"], beta=w["beta"], a="1-bit 2:4 prepared",
+                    b="fp16 N(0,1)", accumulate="fp32", d="fp16"),
+        roofline=dict(bound="mfma", achieved=tflops, peak=SMFMAC_PEAK_TFLOPS, unit="TFLOP/s",
+                      frac=tflops / SMFMAC_PEAK_TFLOPS, traffic=None,
+                      note="dense-equivalent FLOPs 2MNK against the fp16 SMFMAC rate (2 x the dense fp16 MFMA peak "
+                           f"{DENSE_F16_PEAK_TFLOPS:.1f}); the same fraction as executed FLOPs MNK against the dense peak",
+                      hbm_gbps_algorithmic=algorithmic_bytes(m, n, k, w["beta"]) / kernel_s / 1e9),
+        wall_ms_per_step=wall_s * 1e3)
+    if not args.no_decode:
+        line["decode_n16"] = run_decode_rotating(11008, 4096, 16)
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(w, operands)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

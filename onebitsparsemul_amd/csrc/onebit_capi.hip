@@ -212,3 +212,12 @@ void onebit_sparse_matmul(void* a, void* b, void* c, void* d, void* e, int m, in
 }
 
 }  // extern "C"
+
+// The reference header declares the entry point without extern "C" (include/onebit_sparse_tensor.h:5), so
+// objects compiled against it reference the C++-mangled name; export that name as well.
+void onebit_sparse_matmul_cxx_name(void* a, void* b, void* c, void* d, void* e, int m, int n, int k)
+    __asm__("_Z20onebit_sparse_matmulPvS_S_S_S_iii");
+__attribute__((visibility("default"))) void onebit_sparse_matmul_cxx_name(void* a, void* b, void* c, void* d, void* e,
+                                                                          int m, int n, int k) {
+  onebit_sparse_matmul(a, b, c, d, e, m, n, k);
+}

@@ -175,3 +175,25 @@ def blas_matmul(a_dense, b_half, c=None, alpha=1.0, beta=0.0, dtype=np.float64):
     if c is not None and beta != 0.0:
         out = out + dtype(beta) * c.astype(dtype)
     return out
+
+
+def cpu_baseline_gemm(a, b_half, e, m, n, k, row_begin, row_end, layout=LAYOUT_REFERENCE, threads=None):
+    """The reference's CPU path (onebit_sparse_mul/__init__.py:67-97: decompress the weight, then a dense
+    torch.matmul) on rows [row_begin, row_end) of A, in fp32 on the host's cores. Returns (seconds of the
+    matmul, seconds of the decompression, result slab as float32 numpy)."""
+    import time
+
+    import torch
+
+    if threads:
+        torch.set_num_threads(threads)
+    t0 = time.perf_counter()
+    dense = decompress_operands(a, e, m, k, layout)[row_begin:row_end]
+    t1 = time.perf_counter()
+    a_t = torch.from_numpy(dense).to(torch.float32)
+    b_t = torch.from_numpy(np.ascontiguousarray(b_half)).to(torch.float32)
+    torch.matmul(a_t[:64], b_t)  # warm-up of the BLAS threads
+    t2 = time.perf_counter()
+    out = torch.matmul(a_t, b_t)
+    t3 = time.perf_counter()
+    return t3 - t2, t1 - t0, out.numpy()

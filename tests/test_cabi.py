@@ -1,0 +1,108 @@
+"""The C ABI of libonebitmul.so as far as it can be exercised without a GPU: the library loads, exports every
+symbol that include/onebit_sparse_tensor.h declares, validates its arguments and reports HIP failures as
+status codes (or, for the 8-argument symbol, as exit(EXIT_FAILURE) like the reference)."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "onebit_sparse_tensor.h")
+
+from onebitsparsemul_amd import _native  # noqa: E402
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(onebit_sparse_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_native.LIB_PATH)
+    declared = _declared_functions()
+    assert "onebit_sparse_matmul" in declared and len(declared) >= 8
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in the header but not exported"
+    assert sorted(_native.EXPORTS) == declared
+    # objects compiled against the reference's C++ header link against the mangled name
+    assert hasattr(lib, "_Z20onebit_sparse_matmulPvS_S_S_S_iii")
+
+
+def test_header_is_plain_c():
+    src = '#include "onebit_sparse_tensor.h"\nint main(void){return onebit_sparse_prepared_bytes(64,32)==0;}\n'
+    out = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-I", os.path.join(ROOT, "include"),
+                          "-x", "c", "-"], input=src.encode(), capture_output=True)
+    assert out.returncode == 0, out.stderr.decode()
+
+
+def test_prepared_bytes():
+    lib = _native.lib()
+    assert lib.onebit_sparse_prepared_bytes(64, 32) == 2 * 1 * 1536
+    assert lib.onebit_sparse_prepared_bytes(8192, 8192) == 8192 * 8192 * 3 // 16   # 1.5 bits per weight
+    assert lib.onebit_sparse_prepared_bytes(11008, 4096) == 11008 * 4096 * 3 // 16
+    assert lib.onebit_sparse_prepared_bytes(0, 32) == 0
+
+
+@pytest.mark.parametrize("m,n,k", [(10, 10, 10), (64, 8, 16), (32, 8, 32), (64, 0, 32), (-64, 8, 32), (64, 8, 48)])
+def test_shape_validation(m, n, k):
+    lib = _native.lib()
+    fake = ctypes.c_void_p(0x1000)
+    rc = lib.onebit_sparse_matmul_ex(fake, fake, fake, fake, fake, m, n, k, 1.0, 0.0, 0, 0, 0, None)
+    assert rc == 1
+    assert _native.last_error() != ""
+    rc = lib.onebit_sparse_matmul_prepared(fake, fake, fake, fake, m, n, k, 1.0, 0.0, 0, 0, None)
+    assert rc == 1
+
+
+def test_argument_validation():
+    lib = _native.lib()
+    fake = ctypes.c_void_p(0x1000)
+    assert lib.onebit_sparse_matmul_ex(None, fake, fake, fake, fake, 64, 8, 32, 1.0, 0.0, 0, 0, 0, None) == 1
+    assert lib.onebit_sparse_matmul_ex(fake, fake, None, fake, fake, 64, 8, 32, 1.0, 1.0, 0, 0, 0, None) == 1  # beta, no C
+    assert lib.onebit_sparse_matmul_ex(fake, fake, fake, fake, fake, 64, 8, 32, 1.0, 0.0, 2, 0, 0, None) == 1   # dtype
+    assert lib.onebit_sparse_matmul_ex(fake, fake, fake, fake, fake, 64, 8, 32, 1.0, 0.0, 0, 0, 7, None) == 1   # layout
+    assert lib.onebit_sparse_prepare(fake, fake, 64, 32, 0, None, None) == 1
+    assert lib.onebit_sparse_prepare(fake, fake, 64, 32, 3, fake, None) == 1
+    assert "layout" in _native.last_error()
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="needs a host without a GPU (pointers are fake)")
+def test_no_device_is_reported_not_fatal():
+    lib = _native.lib()
+    fake = ctypes.c_void_p(0x1000)
+    rc = lib.onebit_sparse_matmul_ex(fake, fake, fake, fake, fake, 64, 8, 32, 1.0, 0.0, 0, 0, 0, None)
+    assert rc == 2
+    assert "HIP error" in _native.last_error()
+
+
+def test_legacy_symbol_exits_on_error():
+    """csrc/kernel_lib.cu:11-20: print one line to stderr and exit(EXIT_FAILURE)."""
+    code = ("import ctypes,sys; L=ctypes.CDLL(sys.argv[1]); p=ctypes.c_void_p(0x1000);"
+            "L.onebit_sparse_matmul(p,p,p,p,p,10,10,10); print('survived')")
+    out = subprocess.run([sys.executable, "-c", code, _native.LIB_PATH], capture_output=True, text=True)
+    assert out.returncode == 1
+    assert "survived" not in out.stdout
+    assert "onebit_sparse_matmul error" in out.stderr
+
+
+def test_python_wrappers_reject_host_tensors():
+    a = torch.zeros(16, 8, dtype=torch.uint8)
+    meta = torch.zeros(64, 2, dtype=torch.int16)
+    with pytest.raises(ValueError):
+        _native.prepare(a, meta, 64, 32)
+
+
+def test_binding_module_loads_and_validates():
+    from onebitsparsemul_amd import onebit_sparse_cuda
+    assert onebit_sparse_cuda.onebit_mul.__doc__.strip().endswith("A32 = Sparse W1 * A16 matmul.")
+    a = torch.zeros(16, 8, dtype=torch.uint8)
+    b = torch.zeros(32, 8, dtype=torch.float16)
+    meta = torch.zeros(64, 2, dtype=torch.int16)
+    c = torch.zeros(64, 8, dtype=torch.float32)
+    with pytest.raises(RuntimeError):
+        onebit_sparse_cuda.onebit_mul(a, b, meta, c)  # host tensors are rejected, nothing is computed on the CPU
