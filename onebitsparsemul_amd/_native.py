@@ -14,7 +14,7 @@ META_REFERENCE, META_CUTLASS, META_LOGICAL = 0, 1, 2
 EXPORTS = (
     "onebit_sparse_matmul", "onebit_sparse_matmul_ex", "onebit_sparse_prepared_bytes", "onebit_sparse_prepare",
     "onebit_sparse_matmul_prepared", "onebit_sparse_last_error", "onebit_sparse_set_tile_config",
-    "onebit_sparse_set_skinny_enabled",
+    "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows",
 )
 
 _lib = None
@@ -43,6 +43,8 @@ def lib():
         L.onebit_sparse_set_tile_config.argtypes = [i32]
         L.onebit_sparse_set_skinny_enabled.restype = None
         L.onebit_sparse_set_skinny_enabled.argtypes = [i32]
+        L.onebit_sparse_set_skinny_rows.restype = None
+        L.onebit_sparse_set_skinny_rows.argtypes = [i32]
         _lib = L
     return _lib
 
@@ -138,3 +140,7 @@ def set_tile_config(cfg):
 
 def set_skinny_enabled(flag):
     lib().onebit_sparse_set_skinny_enabled(1 if flag else 0)
+
+
+def set_skinny_rows(rows):
+    lib().onebit_sparse_set_skinny_rows(rows)

@@ -17,6 +17,7 @@ namespace {
 thread_local std::string g_last_error;
 std::atomic<int> g_tile_config{-1};
 std::atomic<int> g_skinny_enabled{1};
+std::atomic<int> g_skinny_rows{-1};
 
 int fail(int code, const char* fmt, ...) {
   char buf[512];
@@ -37,21 +38,16 @@ int fail(int code, const char* fmt, ...) {
 
 constexpr int kMaxDevices = 64;
 
-// Library-owned device memory: the reordered operand of the one-call entry points, the split-K partial
-// sums and the arrival counters of the skinny kernel. Grow-only, one set per device, freed at process exit
-// by the runtime. Work that uses it is ordered by the caller's stream.
+// Library-owned device memory: the reordered operand of the one-call entry points. Grow-only, one per
+// device, freed at process exit by the runtime. Work that uses it is ordered by the caller's stream.
 struct DeviceState {
   std::mutex mu;
   void* prep = nullptr;
   size_t prep_bytes = 0;
-  float* partials = nullptr;
-  size_t partial_bytes = 0;
-  int* counters = nullptr;
-  size_t counter_count = 0;
 };
 DeviceState g_dev[kMaxDevices];
 
-int grow(void** ptr, size_t* have, size_t need, bool zero, hipStream_t stream) {
+int grow(void** ptr, size_t* have, size_t need) {
   if (need <= *have) return ONEBIT_OK;
   if (*ptr) {
     // earlier work on any stream may still read the old buffer
@@ -62,7 +58,6 @@ int grow(void** ptr, size_t* have, size_t need, bool zero, hipStream_t stream) {
   }
   const size_t bytes = (need + 4095) & ~size_t(4095);
   ONEBIT_HIP(hipMalloc(ptr, bytes));
-  if (zero) ONEBIT_HIP(hipMemsetAsync(*ptr, 0, bytes, stream));
   *have = bytes;
   return ONEBIT_OK;
 }
@@ -96,11 +91,7 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
   if (beta != 0.f && !c) return fail(ONEBIT_ERR_ARGUMENT, "c must not be null when beta != 0");
   const int kc_total = (k + onebit::kChunkK - 1) / onebit::kChunkK;
 
-  if (n <= 32 && g_skinny_enabled.load()) {
-    int device = 0;
-    ONEBIT_HIP(hipGetDevice(&device));
-    if (device < 0 || device >= kMaxDevices) return fail(ONEBIT_ERR_HIP, "device index %d out of range", device);
-    DeviceState& ds = g_dev[device];
+  if (n <= onebit::kSkinnyMaxN && g_skinny_enabled.load()) {
     onebit::SkinnyArgs args{};
     args.prep = static_cast<const uint8_t*>(prepared);
     args.b = static_cast<const _Float16*>(b);
@@ -111,24 +102,9 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
     args.alpha = alpha; args.beta = beta;
     args.c_f16 = c_dtype == ONEBIT_DTYPE_F16;
     args.d_f16 = d_dtype == ONEBIT_DTYPE_F16;
-    const int sk = onebit::skinny_pick_sk(m, k);
-    args.splits = (kc_total + sk - 1) / sk;
-    {
-      std::lock_guard<std::mutex> lock(ds.mu);
-      if (args.splits > 1) {
-        const int row_groups = (m + onebit::skinny_rows_per_group() - 1) / onebit::skinny_rows_per_group();
-        int rc = grow(reinterpret_cast<void**>(&ds.partials), &ds.partial_bytes,
-                      (size_t)args.splits * m * n * sizeof(float), false, stream);
-        if (rc) return rc;
-        size_t counter_bytes = ds.counter_count * sizeof(int);
-        rc = grow(reinterpret_cast<void**>(&ds.counters), &counter_bytes, (size_t)row_groups * sizeof(int), true, stream);
-        if (rc) return rc;
-        ds.counter_count = counter_bytes / sizeof(int);
-      }
-      args.partials = ds.partials;
-      args.counters = ds.counters;
-    }
-    ONEBIT_HIP(onebit::launch_skinny(args, sk, stream));
+    int rows = g_skinny_rows.load();
+    if (rows <= 0) rows = (m / 64 >= 256) ? 64 : 32;  // enough workgroups to cover the 256 CUs
+    ONEBIT_HIP(onebit::launch_skinny(args, rows, stream));
     return ONEBIT_OK;
   }
 
@@ -154,6 +130,7 @@ const char* onebit_sparse_last_error(void) { return g_last_error.c_str(); }
 
 void onebit_sparse_set_tile_config(int tile_config) { g_tile_config.store(tile_config); }
 void onebit_sparse_set_skinny_enabled(int enabled) { g_skinny_enabled.store(enabled ? 1 : 0); }
+void onebit_sparse_set_skinny_rows(int rows) { g_skinny_rows.store(rows); }
 
 size_t onebit_sparse_prepared_bytes(int m, int k) {
   if (m <= 0 || k <= 0) return 0;
@@ -195,7 +172,7 @@ int onebit_sparse_matmul_ex(const void* a, const void* b, const void* c, void* d
   void* prep = nullptr;
   {
     std::lock_guard<std::mutex> lock(ds.mu);
-    if (int rc = grow(&ds.prep, &ds.prep_bytes, onebit::prepared_bytes(m, k), false, s)) return rc;
+    if (int rc = grow(&ds.prep, &ds.prep_bytes, onebit::prepared_bytes(m, k))) return rc;
     prep = ds.prep;
   }
   ONEBIT_HIP(onebit::launch_prepare(a, e, prep, m, k, meta_layout, s));

@@ -351,59 +351,26 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 }
 
 // =====================================================================================================
-// skinny_kernel: N <= 32 (decode shapes). HBM-bound: every byte of the prepared operand is read once.
-// Workgroup = 4 wavefronts sharing one K slice (SK chunks of 256) of B, staged into LDS as a zero-padded
-// [k][NC]-image; wavefront w owns R row blocks (32 rows each). grid = (row groups, K splits).
-// With more than one K split, partial sums go to a workspace and the last workgroup to finish a row group
-// adds them in split order (deterministic) and applies the epilogue.
+// skinny_kernel: N <= 16 (decode shapes). HBM-bound: every byte of the prepared operand is read once.
+// Workgroup = 16 wavefronts that share R row blocks (32 rows each) and split K among themselves: wavefront w
+// takes the K chunks (of 256) w, w+16, w+32, ... Each wavefront stages the B rows of its chunk in a private
+// 8 KiB LDS region as a zero-padded [256][16] fp16 image, feeds them to SMFMAC through transpose reads and
+// keeps a 32x32 fp32 partial tile per row block. The sixteen partial tiles are added through LDS in
+// wavefront order (deterministic) and the epilogue is applied. grid = M / (32 R) workgroups; no global
+// workspace, no atomics.
 // =====================================================================================================
-template <int R, int SK, int NC>
-__global__ __launch_bounds__(256) void skinny_kernel(SkinnyArgs p) {
-  constexpr int RS = NC * 2;  // bytes per LDS row
-  __shared__ __attribute__((aligned(16))) char bs[SK * kChunkK * RS];
-  __shared__ int last_flag;
+constexpr int kSkinnyWaves = 16;
+constexpr int kSkinnyRegion = kChunkK * 16 * 2;  // bytes of one wavefront's B image
+
+template <int R>
+__global__ __launch_bounds__(1024) void skinny_kernel(SkinnyArgs p) {
+  static_assert(R * 32 * 16 * 4 <= kSkinnyRegion, "partial tiles must fit the wavefront's LDS region");
+  __shared__ __attribute__((aligned(16))) char bs[kSkinnyWaves * kSkinnyRegion];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int rg = blockIdx.x, split = blockIdx.y;
-  const int kc0 = split * SK;
   const int rb_total = p.m / kRowBlock;
-  const int rb_first = (rg * 4 + wave) * R;
-
-  // weight stream first: all requests of this wavefront are in flight while B is staged
-  AChunk a[SK][R];
-#pragma unroll
-  for (int c = 0; c < SK; ++c) {
-    int kc = kc0 + c;
-    if (kc >= p.kc_total) kc = p.kc_total - 1;  // valid address; its B rows are zero
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      int rb = rb_first + r;
-      if (rb >= rb_total) rb = rb_total - 1;
-      a[c][r] = load_a_chunk(p.prep + ((size_t)rb * p.kc_total + kc) * kBlockBytes, lane);
-    }
-  }
-
-  // stage B rows [kc0*256, +SK*256) x NC columns, zero outside the matrix
-  {
-    const int k_base = kc0 * kChunkK;
-    if (NC == 16 && p.n == 16 && (reinterpret_cast<uintptr_t>(p.b) & 15) == 0) {
-      const u32x4_t* src = reinterpret_cast<const u32x4_t*>(p.b + (size_t)k_base * 16);
-      for (int idx = tid; idx < SK * kChunkK * 2; idx += 256) {
-        const int row = idx >> 1;
-        u32x4_t v = {0, 0, 0, 0};
-        if (k_base + row < p.k) v = src[idx];
-        *reinterpret_cast<u32x4_t*>(bs + idx * 16) = v;
-      }
-    } else {
-      for (int idx = tid; idx < SK * kChunkK * NC; idx += 256) {
-        const int row = idx / NC, col = idx % NC;
-        _Float16 v = (_Float16)0.f;
-        if (k_base + row < p.k && col < p.n) v = p.b[(size_t)(k_base + row) * p.n + col];
-        *reinterpret_cast<_Float16*>(bs + row * RS + col * 2) = v;
-      }
-    }
-  }
-  __syncthreads();
+  const int rb_first = blockIdx.x * R;
+  char* region = bs + wave * kSkinnyRegion;
 
   float16_t acc[R];
 #pragma unroll
@@ -412,24 +379,69 @@ __global__ __launch_bounds__(256) void skinny_kernel(SkinnyArgs p) {
     for (int v = 0; v < 16; ++v) acc[r][v] = 0.f;
 
   const int i16 = lane & 15, gb = lane >> 5;
-  const int half32 = (NC == 32) ? ((lane & 31) >> 4) : 0;  // NC == 16: lanes 16-31 duplicate columns 0-15
-  const char* lane_ptr = bs + (8 * gb + (i16 >> 2)) * RS + ((i16 & 3) + 4 * half32) * 8;
+  // lanes 16-31 and 48-63 would hold columns 16-31: they re-read columns 0-15 and are never stored
+  const char* lane_ptr = region + (8 * gb + (i16 >> 2)) * 32 + (i16 & 3) * 8;
+  const bool vector_b = p.n == 16 && (reinterpret_cast<uintptr_t>(p.b) & 15) == 0;
 
+  for (int kc = wave; kc < p.kc_total; kc += kSkinnyWaves) {
+    AChunk a[R];
 #pragma unroll
-  for (int c = 0; c < SK; ++c) {
+    for (int r = 0; r < R; ++r) {
+      int rb = rb_first + r;
+      if (rb >= rb_total) rb = rb_total - 1;
+      a[r] = load_a_chunk(p.prep + ((size_t)rb * p.kc_total + kc) * kBlockBytes, lane);
+    }
+    const int k_base = kc * kChunkK;
+    const int rows_valid = (p.k - k_base) < kChunkK ? (p.k - k_base) : kChunkK;  // >= 1
+    if (vector_b) {
+      // the chunk's rows are 8 KiB of consecutive memory: eight 16-byte pieces per lane
+      const u32x4_t* src = reinterpret_cast<const u32x4_t*>(p.b + (size_t)k_base * 16);
+      u32x4_t v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int idx = lane + i * 64;
+        const bool ok = (idx >> 1) < rows_valid;
+        v[i] = src[ok ? idx : 0];
+        if (!ok) v[i] = u32x4_t{0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4_t*>(region + (lane + i * 64) * 16) = v[i];
+    } else {
+      // any n <= 16, any alignment: the valid part of the chunk is one run of rows_valid * n elements
+#pragma unroll
+      for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4_t*>(region + (lane + i * 64) * 16) = u32x4_t{0, 0, 0, 0};
+      const _Float16* src = p.b + (size_t)k_base * p.n;
+      const int total = rows_valid * p.n;
+      constexpr int BATCH = 8;
+      for (int e0 = lane; e0 < total; e0 += 64 * BATCH) {
+        _Float16 v[BATCH];
+#pragma unroll
+        for (int i = 0; i < BATCH; ++i) {
+          const int e = e0 + i * 64;
+          v[i] = src[e < total ? e : 0];
+        }
+#pragma unroll
+        for (int i = 0; i < BATCH; ++i) {
+          const int e = e0 + i * 64;
+          if (e < total) *reinterpret_cast<_Float16*>(region + (e / p.n) * 32 + (e % p.n) * 2) = v[i];
+        }
+      }
+    }
+    // the region is private to this wavefront and its LDS operations execute in order: no barrier needed
+
     auto step = [&](auto step_tag) {
       constexpr int STEP = decltype(step_tag)::value;
       u32x8_t raw;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int row_const = c * kChunkK + STEP * 32 + 4 * (q & 1) + 16 * (q >> 1);
-        const u32x2_t t = lds_read_tr16(lane_ptr + row_const * RS);
+        const int row_const = STEP * 32 + 4 * (q & 1) + 16 * (q >> 1);
+        const u32x2_t t = lds_read_tr16(lane_ptr + row_const * 32);
         raw[2 * q] = t.x;
         raw[2 * q + 1] = t.y;
       }
       const half16_t bv = __builtin_bit_cast(half16_t, raw);
 #pragma unroll
-      for (int r = 0; r < R; ++r) acc[r] = smfmac_step<STEP>(a[c][r], expand_signs<STEP>(a[c][r]), bv, acc[r]);
+      for (int r = 0; r < R; ++r) acc[r] = smfmac_step<STEP>(a[r], expand_signs<STEP>(a[r]), bv, acc[r]);
     };
     step(std::integral_constant<int, 0>{});
     step(std::integral_constant<int, 1>{});
@@ -441,60 +453,38 @@ __global__ __launch_bounds__(256) void skinny_kernel(SkinnyArgs p) {
     step(std::integral_constant<int, 7>{});
   }
 
-  const int col = lane & 31;
-  const int row_lane = 4 * (lane >> 5);
-  const bool col_ok = col < p.n && (NC == 32 || (lane & 31) < 16);
-  auto store_out = [&](size_t o, float sum) {
-    float x = p.alpha * sum;
-    if (p.beta != 0.f) {
-      const float cv = p.c_f16 ? (float)reinterpret_cast<const _Float16*>(p.c)[o] : reinterpret_cast<const float*>(p.c)[o];
-      x = x + p.beta * cv;
+  // ---- add the sixteen partial tiles through LDS: region of wavefront w := its R tiles as [r][32 rows][16 cols] fp32
+  {
+    float* tile = reinterpret_cast<float*>(region);
+    const int col = lane & 31;
+    if (col < 16) {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int row = 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+          tile[(r * 32 + row) * 16 + col] = acc[r][v];
+        }
     }
-    if (p.d_f16) reinterpret_cast<_Float16*>(p.d)[o] = (_Float16)x;
-    else reinterpret_cast<float*>(p.d)[o] = x;
-  };
-
-  if (p.splits == 1) {
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int row = (rb_first + r) * kRowBlock + 8 * (v / 4) + row_lane + (v % 4);
-        if (col_ok && row < p.m) store_out((size_t)row * p.n + col, acc[r][v]);
-      }
-    return;
-  }
-
-  // ---- split-K: publish the partial tile, the last workgroup of the row group reduces ----
-  float* part = p.partials + (size_t)split * p.m * p.n;
-#pragma unroll
-  for (int r = 0; r < R; ++r)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int row = (rb_first + r) * kRowBlock + 8 * (v / 4) + row_lane + (v % 4);
-      if (col_ok && row < p.m) part[(size_t)row * p.n + col] = acc[r][v];
-    }
-  __threadfence();  // make the partial tile visible device-wide before the arrival count
-  __syncthreads();
-  if (tid == 0) {
-    const int prev = __hip_atomic_fetch_add(&p.counters[rg], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    last_flag = (prev == p.splits - 1);
   }
   __syncthreads();
-  if (!last_flag) return;
-  __threadfence();
-  const int rows_per_group = 4 * R * kRowBlock;
-  const int row_begin = rg * rows_per_group;
-  const int row_end = (row_begin + rows_per_group < p.m) ? row_begin + rows_per_group : p.m;
-  const int count = (row_end - row_begin) * p.n;
-  const size_t base = (size_t)row_begin * p.n;
-  const size_t split_stride = (size_t)p.m * p.n;
-  for (int idx = tid; idx < count; idx += 256) {
+  for (int idx = tid; idx < R * 32 * 16; idx += 1024) {
     float sum = 0.f;
-    for (int s = 0; s < p.splits; ++s) sum += __builtin_nontemporal_load(p.partials + s * split_stride + base + idx);
-    store_out(base + idx, sum);
+#pragma unroll
+    for (int w = 0; w < kSkinnyWaves; ++w) sum += reinterpret_cast<const float*>(bs + w * kSkinnyRegion)[idx];
+    const int col = idx & 15;
+    const int row = rb_first * kRowBlock + (idx >> 4);
+    if (col < p.n && row < p.m) {
+      const size_t o = (size_t)row * p.n + col;
+      float x = p.alpha * sum;
+      if (p.beta != 0.f) {
+        const float cv = p.c_f16 ? (float)reinterpret_cast<const _Float16*>(p.c)[o] : reinterpret_cast<const float*>(p.c)[o];
+        x = x + p.beta * cv;
+      }
+      if (p.d_f16) reinterpret_cast<_Float16*>(p.d)[o] = (_Float16)x;
+      else reinterpret_cast<float*>(p.d)[o] = x;
+    }
   }
-  if (tid == 0) __hip_atomic_store(&p.counters[rg], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next call
 }
 
 // =====================================================================================================
@@ -539,33 +529,18 @@ hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
   }
 }
 
-template <int R, int SK, int NC>
+template <int R>
 static hipError_t launch_skinny_cfg(const SkinnyArgs& args, hipStream_t stream) {
-  const int row_groups = (args.m + 4 * R * kRowBlock - 1) / (4 * R * kRowBlock);
-  hipLaunchKernelGGL((skinny_kernel<R, SK, NC>), dim3(row_groups, args.splits), dim3(256), 0, stream, args);
+  const int row_blocks = args.m / kRowBlock;
+  hipLaunchKernelGGL((skinny_kernel<R>), dim3((row_blocks + R - 1) / R), dim3(1024), 0, stream, args);
   return hipGetLastError();
 }
 
-int skinny_rows_per_group() { return 4 * 2 * kRowBlock; }
-
-int skinny_pick_sk(int m, int k) {
-  const int row_groups = (m + skinny_rows_per_group() - 1) / skinny_rows_per_group();
-  const int kc_total = (k + kChunkK - 1) / kChunkK;
-  const int cand[4] = {8, 4, 2, 1};
-  for (int i = 0; i < 4; ++i) {
-    const int sk = cand[i];
-    if (row_groups * ((kc_total + sk - 1) / sk) >= 256) return sk;
-  }
-  return 1;
-}
-
-hipError_t launch_skinny(SkinnyArgs args, int sk, hipStream_t stream) {
-  const bool wide = args.n > 16;
-  switch (sk) {
-    case 1: return wide ? launch_skinny_cfg<2, 1, 32>(args, stream) : launch_skinny_cfg<2, 1, 16>(args, stream);
-    case 2: return wide ? launch_skinny_cfg<2, 2, 32>(args, stream) : launch_skinny_cfg<2, 2, 16>(args, stream);
-    case 4: return wide ? launch_skinny_cfg<2, 4, 32>(args, stream) : launch_skinny_cfg<2, 4, 16>(args, stream);
-    case 8: return wide ? launch_skinny_cfg<2, 8, 32>(args, stream) : launch_skinny_cfg<2, 8, 16>(args, stream);
+hipError_t launch_skinny(SkinnyArgs args, int rows_per_group, hipStream_t stream) {
+  switch (rows_per_group) {
+    case 32: return launch_skinny_cfg<1>(args, stream);
+    case 64: return launch_skinny_cfg<2>(args, stream);
+    case 128: return launch_skinny_cfg<4>(args, stream);
     default: return hipErrorInvalidValue;
   }
 }

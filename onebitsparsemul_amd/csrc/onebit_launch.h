@@ -22,11 +22,8 @@ struct SkinnyArgs {
   const _Float16* b;
   const void* c;
   void* d;
-  float* partials;  // splits x m x n fp32 (unused when splits == 1)
-  int* counters;    // one arrival counter per row group, zero between calls
   int m, n, k;
   int kc_total;
-  int splits;       // ceil(kc_total / SK)
   float alpha, beta;
   int c_f16, d_f16;
 };
@@ -36,9 +33,8 @@ enum TileConfig { kTile512x128 = 0, kTile256x128 = 1, kTile128x128 = 2, kTile256
 hipError_t launch_prepare(const void* a, const void* e, void* prep, int m, int k, int layout, hipStream_t stream);
 hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream);
 
-// Split-K kernel for n <= 32. sk = K chunks (of 256) per workgroup, one of 1, 2, 4, 8.
-int skinny_rows_per_group();
-int skinny_pick_sk(int m, int k);
-hipError_t launch_skinny(SkinnyArgs args, int sk, hipStream_t stream);
+// Split-K kernel for n <= 16; rows_per_group (32, 64 or 128) = weight rows one workgroup covers.
+constexpr int kSkinnyMaxN = 16;
+hipError_t launch_skinny(SkinnyArgs args, int rows_per_group, hipStream_t stream);
 
 }  // namespace onebit
