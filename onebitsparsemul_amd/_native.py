@@ -6,7 +6,8 @@ import os
 import torch
 
 _DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_DIR, "libonebitmul.so")
+# ONEBITMUL_LIBRARY overrides the in-tree build (e.g. to try an experimental build of the same ABI).
+LIB_PATH = os.environ.get("ONEBITMUL_LIBRARY") or os.path.join(_DIR, "libonebitmul.so")
 
 F32, F16 = 0, 1
 META_REFERENCE, META_CUTLASS, META_LOGICAL = 0, 1, 2

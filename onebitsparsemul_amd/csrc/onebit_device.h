@@ -71,15 +71,24 @@ __device__ __forceinline__ AChunk load_a_chunk_lds(const char* block, int lane) 
   return r;
 }
 
-// Expand the eight +-1 values of K step `STEP` (0..7, compile time) into four packed fp16 registers.
+// fp16 1.0 in both halves, held in a vector register: v_and_or_b32 can then take the sign mask as its only
+// literal operand (two literals in one instruction are not encodable, and cost a third instruction).
+__device__ __forceinline__ uint32_t packed_one_in_vgpr() {
+  uint32_t one = 0x3C003C00u;
+  asm volatile("" : "+v"(one));
+  return one;
+}
+
+// Expand the eight +-1 values of K step `STEP` (0..7, compile time) into four packed fp16 registers:
+// two instructions per register (shift, and-or).
 template <int STEP>
-__device__ __forceinline__ half8_t expand_signs(const AChunk& a) {
+__device__ __forceinline__ half8_t expand_signs(const AChunk& a, uint32_t packed_one) {
   const uint32_t w = STEP < 4 ? a.sign.x : a.sign.y;
   u32x4_t v;
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
     const int j = 4 * (STEP % 4) + p;
-    v[p] = ((w << j) & 0x80008000u) | 0x3C003C00u;  // fp16 1.0 with the stored sign
+    v[p] = ((w << j) & 0x80008000u) | packed_one;  // fp16 1.0 with the stored sign
   }
   return __builtin_bit_cast(half8_t, v);
 }
@@ -109,11 +118,25 @@ __device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_wave_ba
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_wave_base), "v"(gptr) : "memory");
 }
 
+// Same copy with the address split into a wave-uniform 64-bit base (scalar registers) and a per-lane 32-bit
+// byte offset: one vector register per copy instead of two, and the base advances with scalar arithmetic.
+__device__ __forceinline__ void lds_dma16_base(const void* base, uint32_t lane_offset, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_wave_base), "v"(lane_offset), "s"(base)
+               : "memory");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter on gfx9");
   // simm16: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]; other counters left open.
   __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8) | ((N >> 4) << 14));
+}
+
+// Same, and additionally waits for every outstanding LDS operation of the wavefront (lgkmcnt = 0).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_lgkm0() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter on gfx9");
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0x0 << 8) | ((N >> 4) << 14));
 }
 
 __device__ __forceinline__ uint32_t lds_offset_of(const void* p) {

@@ -116,7 +116,7 @@ __device__ __forceinline__ void tile_of_block(int b, int tiles_m, int tiles_n, i
 // One stage (64 K = two SMFMAC K steps) of a wavefront's FM x FN tile.
 template <int FM, int FN, int BN, int STAGE_IN_CHUNK>
 __device__ __forceinline__ void compute_stage(const char* stage_lds, const AChunk (&a)[FM], float16_t (&acc)[FM][FN],
-                                              const int (&frag_off)[FN], int lane_row_off) {
+                                              const int (&frag_off)[FN], int lane_row_off, uint32_t one) {
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks) {
     constexpr int dummy = 0;
@@ -137,8 +137,8 @@ __device__ __forceinline__ void compute_stage(const char* stage_lds, const AChun
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm) {
       half8_t av;
-      if (ks == 0) av = expand_signs<2 * STAGE_IN_CHUNK>(a[fm]);
-      else av = expand_signs<2 * STAGE_IN_CHUNK + 1>(a[fm]);
+      if (ks == 0) av = expand_signs<2 * STAGE_IN_CHUNK>(a[fm], one);
+      else av = expand_signs<2 * STAGE_IN_CHUNK + 1>(a[fm], one);
 #pragma unroll
       for (int fn = 0; fn < FN; ++fn) {
         if (ks == 0) acc[fm][fn] = smfmac_step<2 * STAGE_IN_CHUNK>(a[fm], av, bv[fn], acc[fm][fn]);
@@ -148,8 +148,76 @@ __device__ __forceinline__ void compute_stage(const char* stage_lds, const AChun
   }
 }
 
+// Compile-time experiment switches (all off in the shipped build): each removes one ingredient of the main
+// loop so that its cost can be measured; results are wrong when any of them is set.
+#ifndef ONEBIT_EXP_NO_LDS_READ
+#define ONEBIT_EXP_NO_LDS_READ 0
+#endif
+#ifndef ONEBIT_EXP_NO_EXPAND
+#define ONEBIT_EXP_NO_EXPAND 0
+#endif
+#ifndef ONEBIT_EXP_NO_COPY
+#define ONEBIT_EXP_NO_COPY 0
+#endif
+#ifndef ONEBIT_EXP_COPY_MODE  /* 1: no A copies, 2: no B copies, 3: B copies never advance (always cache hits) */
+#define ONEBIT_EXP_COPY_MODE 0
+#endif
+#ifndef ONEBIT_EXP_NO_BARRIER
+#define ONEBIT_EXP_NO_BARRIER 0
+#endif
+#ifndef ONEBIT_EXP_NO_STORE
+#define ONEBIT_EXP_NO_STORE 0
+#endif
+
+// ---- software-pipelined building blocks of the asynchronous-copy main loop -------------------------
+// B fragments of one 32-wide K step (ks = 0/1 inside a 64-row stage image).
+template <int FN, int BN>
+__device__ __forceinline__ void load_b_frags(const char* stage_lds, int ks, half16_t (&bv)[FN], const int (&frag_off)[FN],
+                                             int lane_row_off) {
+  if (ONEBIT_EXP_NO_LDS_READ) {
+#pragma unroll
+    for (int fn = 0; fn < FN; ++fn) asm volatile("" : "+v"(bv[fn]));
+    return;
+  }
+#pragma unroll
+  for (int fn = 0; fn < FN; ++fn) {
+    u32x8_t raw;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int row_const = ks * 32 + 4 * (q & 1) + 16 * (q >> 1);
+      const u32x2_t t = lds_read_tr16(stage_lds + lane_row_off + row_const * (BN * 2) + frag_off[fn]);
+      raw[2 * q] = t.x;
+      raw[2 * q + 1] = t.y;
+    }
+    bv[fn] = __builtin_bit_cast(half16_t, raw);
+  }
+}
+
+template <int STEP, int FM>
+__device__ __forceinline__ void expand_frags(const AChunk (&a)[FM], uint32_t one, half8_t (&av)[FM]) {
+  if (ONEBIT_EXP_NO_EXPAND) {
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm) asm volatile("" : "+v"(av[fm]));
+    return;
+  }
+#pragma unroll
+  for (int fm = 0; fm < FM; ++fm) av[fm] = expand_signs<STEP>(a[fm], one);
+}
+
+template <int STEP, int FM, int FN>
+__device__ __forceinline__ void mfma_frags(const AChunk (&a)[FM], const half8_t (&av)[FM], const half16_t (&bv)[FN],
+                                           float16_t (&acc)[FM][FN]) {
+#pragma unroll
+  for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+    for (int fn = 0; fn < FN; ++fn) acc[fm][fn] = smfmac_step<STEP>(a[fm], av[fm], bv[fn], acc[fm][fn]);
+}
+
+// Source of zeros for the asynchronous copies of B rows at or past K.
+__device__ __attribute__((aligned(16))) uint32_t g_zero16[4] = {0, 0, 0, 0};
+
 template <int WM, int WN, int FM, int FN, bool DMA>
-__global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
+__global__ __launch_bounds__(256, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmArgs p) {
   using TS = TileShape<WM, WN, FM, FN>;
   constexpr int BM = TS::BM, BN = TS::BN, CH = TS::CH, NL = TS::NL;
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -186,6 +254,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     frag_off[fn] = ((lc ^ chunk_swizzle<BN>(lane_row)) << 4) + (c8 & 1) * 8;
   }
 
+  const uint32_t one = packed_one_in_vgpr();
   float16_t acc[FM][FN];
 #pragma unroll
   for (int fm = 0; fm < FM; ++fm)
@@ -198,9 +267,11 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
   const int chunks = (stages_total + kStages - 1) / kStages;
 
   if constexpr (DMA) {
-    // ---- asynchronous copy pattern for B: NL chunk copies per thread per stage ----
-    // copy i of wavefront w fills LDS slots [(4 i + w) * 64, +64) of the stage; slot s = (row, physical chunk).
-    const char* gsrc[NL];
+    // ---- asynchronous copy pattern for B: NL 16-byte copies per thread per stage ----
+    // copy i of wavefront w fills LDS slots [(4 i + w) * 64, +64) of the stage; slot = (row, physical chunk).
+    // Global address = wave-uniform base of the stage + per-lane byte offset.
+    uint32_t b_off[NL];
+    int copy_row[NL];
     uint32_t lds_dst[NL];
     const uint32_t smem_base = lds_offset_of(smem);
 #pragma unroll
@@ -208,23 +279,33 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
       const int slot = (4 * i + wave) * 64 + lane;
       const int row = slot / CH, pc = slot % CH;
       const int lc = pc ^ chunk_swizzle<BN>(row);
-      int col = n0 + 8 * lc;
-      if (col >= p.n) col = n0;  // columns past N: any valid address will do, the results are not stored
-      gsrc[i] = reinterpret_cast<const char*>(p.b) + ((size_t)row * p.n + col) * 2;
+      int col = 8 * lc;
+      if (n0 + col >= p.n) col = 0;  // columns past N: any valid address will do, the results are not stored
+      b_off[i] = (uint32_t)(row * p.n + col) * 2u;
+      copy_row[i] = row;
       lds_dst[i] = smem_base + (4 * i + wave) * 1024;
     }
+    const char* b_stage = reinterpret_cast<const char*>(p.b) + (size_t)n0 * 2;  // advances one stage per copy
     const size_t stage_stride = (size_t)kStageK * p.n * 2;
-    int next_stage = 0;  // next stage index to copy
+    const char* zeros = reinterpret_cast<const char*>(g_zero16);
+    int next_k0 = 0;  // first K row of the next stage to copy
+    // Rows at or past K are copied from a block of zeros, so stages past the end of K (the ring always runs
+    // whole chunks of four stages) and the padding of the prepared operand contribute nothing, and the
+    // number of copies in flight, which the vmcnt waits rely on, is the same in every iteration.
     auto issue_b = [&](int ring) {
+      if (ONEBIT_EXP_NO_COPY || ONEBIT_EXP_COPY_MODE == 2) return;
+      if (next_k0 + kStageK <= p.k) {  // wave-uniform: a full stage
 #pragma unroll
-      for (int i = 0; i < NL; ++i) lds_dma16(gsrc[i], lds_dst[i] + ring * TS::STAGE_BYTES);
-      // past the last stage the same (valid) rows are copied again so that the number of copies in
-      // flight, which the vmcnt waits below rely on, stays constant
-      if (next_stage + 1 < stages_total) {
+        for (int i = 0; i < NL; ++i) lds_dma16_base(b_stage, b_off[i], lds_dst[i] + ring * TS::STAGE_BYTES);
+      } else {
 #pragma unroll
-        for (int i = 0; i < NL; ++i) gsrc[i] += stage_stride;
+        for (int i = 0; i < NL; ++i) {
+          const char* src = (next_k0 + copy_row[i] < p.k) ? b_stage + b_off[i] : zeros;
+          lds_dma16(src, lds_dst[i] + ring * TS::STAGE_BYTES);
+        }
       }
-      ++next_stage;
+      if (ONEBIT_EXP_COPY_MODE != 3) b_stage += stage_stride;
+      next_k0 += kStageK;
     };
 
     // ---- asynchronous copy pattern for A: the workgroup's BM/32 prepared blocks of one K chunk ----
@@ -232,7 +313,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
     // re-copies the first block into padding so that every wavefront issues the same number of requests).
     constexpr int NA = TS::NA;
     char* a_lds = smem + TS::LDS_B_BYTES;
-    const char* a_src[NA];
+    uint32_t a_off[NA];
     uint32_t a_dst[NA];
     {
       const int rb0 = tile_m * (BM / kRowBlock);
@@ -243,60 +324,86 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
         if (blk >= BM / kRowBlock) blk = 0;
         int rb = rb0 + blk;
         if (rb >= rb_total) rb = rb_total - 1;
-        a_src[j] = reinterpret_cast<const char*>(p.prep) + (size_t)rb * p.kc_total * kBlockBytes + off;
+        a_off[j] = (uint32_t)((size_t)rb * p.kc_total * kBlockBytes + off);  // the launcher checks it fits 32 bits
         a_dst[j] = smem_base + TS::LDS_B_BYTES + (4 * j + wave) * 1024;
       }
     }
+    const char* a_chunk = reinterpret_cast<const char*>(p.prep);  // advances one K chunk per copy
     int next_chunk = 0;
     auto issue_a = [&]() {
+      if (ONEBIT_EXP_NO_COPY || ONEBIT_EXP_COPY_MODE == 1) return;
 #pragma unroll
-      for (int j = 0; j < NA; ++j) lds_dma16(a_src[j], a_dst[j]);
-      if (next_chunk + 1 < chunks) {
-#pragma unroll
-        for (int j = 0; j < NA; ++j) a_src[j] += kBlockBytes;
-      }
+      for (int j = 0; j < NA; ++j) lds_dma16_base(a_chunk, a_off[j], a_dst[j]);
+      if (next_chunk + 1 < chunks) a_chunk += kBlockBytes;  // past the last chunk the last one is copied again
       ++next_chunk;
     };
     const char* a_frag_lds[FM];
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm) a_frag_lds[fm] = a_lds + (wm * FM + fm) * kBlockBytes;
 
-    // Request order: A(0) B(0) B(1) B(2) | per chunk c: s0: B(4c+3)  s1: B(4c+4) A(c+1)  s2: B(4c+5)  s3: B(4c+6)
+    // Software pipeline. One K step (32 wide) is one scheduling region in which the SMFMACs of the step run
+    // while the B fragments and the expanded A of the next step are fetched. The workgroup barrier sits in the
+    // middle of each stage s: it publishes stage s+1 (read right after it) and frees the ring slot of stage s
+    // (all of its reads were issued in the first half), into which stage s+4 is then copied.
+    // Request order: A(0) B(0) B(1) B(2) B(3) | chunk c: mid s0: A(c+1) B(4c+4)  mid s1: B(4c+5)
+    //                                                     mid s2: B(4c+6)        mid s3: B(4c+7)
     issue_a();
 #pragma unroll
-    for (int s = 0; s < kStages - 1; ++s) issue_b(s);
+    for (int s = 0; s < kStages; ++s) issue_b(s);
+
+    AChunk a_cur[FM];
+    half16_t bv0[FN], bv1[FN];
+    half8_t av0[FM], av1[FM];
+    wait_vmcnt<3 * NL>();  // A(0) and B(0) have landed
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm) a_cur[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);
+    load_b_frags<FN, BN>(smem, 0, bv0, frag_off, lane_row_off);
+    expand_frags<0>(a_cur, one, av0);
+
+#define ONEBIT_STAGE(S, WAITCNT, ISSUE_A)                                                                        \
+    {                                                                                                            \
+      load_b_frags<FN, BN>(smem + (S) * TS::STAGE_BYTES, 1, bv1, frag_off, lane_row_off);                         \
+      expand_frags<2 * (S) + 1>(a_cur, one, av1);                                                                \
+      mfma_frags<2 * (S)>(a_cur, av0, bv0, acc);                                                                 \
+      __builtin_amdgcn_sched_barrier(0); /* keep the step's work inside its region */                           \
+      wait_vmcnt_lgkm0<(WAITCNT)>(); /* copies of stage S+1 landed; this wavefront's reads of stage S returned */ \
+      if (!ONEBIT_EXP_NO_BARRIER) __builtin_amdgcn_s_barrier();                                                  \
+      if (ISSUE_A) issue_a();                                                                                    \
+      issue_b(S);                                                                                                \
+      load_b_frags<FN, BN>(smem + (((S) + 1) % kStages) * TS::STAGE_BYTES, 0, bv0, frag_off, lane_row_off);       \
+    }
 
     for (int kc = 0; kc < chunks; ++kc) {
-      AChunk a_cur[FM];
-      // stage 0: needs B(4c) and A(c); newer requests: two B stages
-      wait_vmcnt<2 * NL>();
-      __builtin_amdgcn_s_barrier();
-      issue_b(3);
+      // mid stage 0: waits for B(4c+1); newer requests: B(4c+2), B(4c+3)
+      ONEBIT_STAGE(0, 2 * NL, true)
+      expand_frags<2>(a_cur, one, av0);
+      mfma_frags<1>(a_cur, av1, bv1, acc);
+      __builtin_amdgcn_sched_barrier(0);
+      // mid stage 1: waits for B(4c+2); newer: B(4c+3), A(c+1), B(4c+4)
+      ONEBIT_STAGE(1, 2 * NL + NA, false)
+      expand_frags<4>(a_cur, one, av0);
+      mfma_frags<3>(a_cur, av1, bv1, acc);
+      __builtin_amdgcn_sched_barrier(0);
+      // mid stage 2: waits for B(4c+3); newer: A(c+1), B(4c+4), B(4c+5)
+      ONEBIT_STAGE(2, 2 * NL + NA, false)
+      expand_frags<6>(a_cur, one, av0);
+      mfma_frags<5>(a_cur, av1, bv1, acc);
+      __builtin_amdgcn_sched_barrier(0);
+      // mid stage 3: waits for B(4c+4), which is newer than A(c+1): the next chunk of A is readable after it
+      ONEBIT_STAGE(3, 2 * NL, false)
+      {
+        AChunk a_next[FM];
 #pragma unroll
-      for (int fm = 0; fm < FM; ++fm) a_cur[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);
-      compute_stage<FM, FN, BN, 0>(smem + 0 * TS::STAGE_BYTES, a_cur, acc, frag_off, lane_row_off);
-
-      // stage 1: newer requests: two B stages. All wavefronts have read A(c) before this barrier.
-      wait_vmcnt<2 * NL>();
-      __builtin_amdgcn_s_barrier();
-      issue_b(0);
-      issue_a();
-      if (kc * kStages + 1 < stages_total)
-        compute_stage<FM, FN, BN, 1>(smem + 1 * TS::STAGE_BYTES, a_cur, acc, frag_off, lane_row_off);
-
-      // stage 2: newer requests: two B stages and one A chunk
-      wait_vmcnt<2 * NL + NA>();
-      __builtin_amdgcn_s_barrier();
-      issue_b(1);
-      if (kc * kStages + 2 < stages_total)
-        compute_stage<FM, FN, BN, 2>(smem + 2 * TS::STAGE_BYTES, a_cur, acc, frag_off, lane_row_off);
-
-      wait_vmcnt<2 * NL + NA>();
-      __builtin_amdgcn_s_barrier();
-      issue_b(2);
-      if (kc * kStages + 3 < stages_total)
-        compute_stage<FM, FN, BN, 3>(smem + 3 * TS::STAGE_BYTES, a_cur, acc, frag_off, lane_row_off);
+        for (int fm = 0; fm < FM; ++fm) a_next[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);
+        expand_frags<0>(a_next, one, av0);
+        mfma_frags<7>(a_cur, av1, bv1, acc);
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm) a_cur[fm] = a_next[fm];
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
+#undef ONEBIT_STAGE
     wait_vmcnt<0>();  // drain the copies issued past the end before the LDS is released
   } else {
     // ---- generic path: any N, any K % 32 == 0, any alignment. One stage at a time, element copies. ----
@@ -316,10 +423,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
         }
         __syncthreads();
       };
-      if (kc * kStages + 0 < stages_total) { fill(0); compute_stage<FM, FN, BN, 0>(smem, a_cur, acc, frag_off, lane_row_off); }
-      if (kc * kStages + 1 < stages_total) { fill(1); compute_stage<FM, FN, BN, 1>(smem, a_cur, acc, frag_off, lane_row_off); }
-      if (kc * kStages + 2 < stages_total) { fill(2); compute_stage<FM, FN, BN, 2>(smem, a_cur, acc, frag_off, lane_row_off); }
-      if (kc * kStages + 3 < stages_total) { fill(3); compute_stage<FM, FN, BN, 3>(smem, a_cur, acc, frag_off, lane_row_off); }
+      if (kc * kStages + 0 < stages_total) { fill(0); compute_stage<FM, FN, BN, 0>(smem, a_cur, acc, frag_off, lane_row_off, one); }
+      if (kc * kStages + 1 < stages_total) { fill(1); compute_stage<FM, FN, BN, 1>(smem, a_cur, acc, frag_off, lane_row_off, one); }
+      if (kc * kStages + 2 < stages_total) { fill(2); compute_stage<FM, FN, BN, 2>(smem, a_cur, acc, frag_off, lane_row_off, one); }
+      if (kc * kStages + 3 < stages_total) { fill(3); compute_stage<FM, FN, BN, 3>(smem, a_cur, acc, frag_off, lane_row_off, one); }
     }
   }
 
@@ -334,7 +441,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int row = row0 + fm * 32 + 8 * (v / 4) + row_lane + (v % 4);
-        if (row < p.m && col < p.n) {
+        if (row < p.m && col < p.n && !(ONEBIT_EXP_NO_STORE && acc[fm][fn][v] != 12345.f)) {
           const size_t o = (size_t)row * p.n + col;
           float x = p.alpha * acc[fm][fn][v];
           if (p.beta != 0.f) {
@@ -378,6 +485,7 @@ __global__ __launch_bounds__(1024) void skinny_kernel(SkinnyArgs p) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[r][v] = 0.f;
 
+  const uint32_t one = packed_one_in_vgpr();
   const int i16 = lane & 15, gb = lane >> 5;
   // lanes 16-31 and 48-63 would hold columns 16-31: they re-read columns 0-15 and are never stored
   const char* lane_ptr = region + (8 * gb + (i16 >> 2)) * 32 + (i16 & 3) * 8;
@@ -441,7 +549,7 @@ __global__ __launch_bounds__(1024) void skinny_kernel(SkinnyArgs p) {
       }
       const half16_t bv = __builtin_bit_cast(half16_t, raw);
 #pragma unroll
-      for (int r = 0; r < R; ++r) acc[r] = smfmac_step<STEP>(a[r], expand_signs<STEP>(a[r]), bv, acc[r]);
+      for (int r = 0; r < R; ++r) acc[r] = smfmac_step<STEP>(a[r], expand_signs<STEP>(a[r], one), bv, acc[r]);
     };
     step(std::integral_constant<int, 0>{});
     step(std::integral_constant<int, 1>{});
@@ -518,13 +626,15 @@ static hipError_t launch_gemm_cfg(GemmArgs args, hipStream_t stream) {
 }
 
 hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
-  const bool aligned = (args.n % 8 == 0) && (args.k % kStageK == 0) && ((reinterpret_cast<uintptr_t>(args.b) & 15) == 0);
+  if (prepared_bytes(args.m, args.k) >= (size_t(1) << 32)) return hipErrorInvalidValue;  // 32-bit copy offsets
+  const bool aligned = (args.n % 8 == 0) && ((reinterpret_cast<uintptr_t>(args.b) & 15) == 0);
   if (!aligned) return launch_gemm_cfg<4, 1, 1, 4, false>(args, stream);
   switch (tile_config) {
     case kTile512x128: return launch_gemm_cfg<4, 1, 4, 4, true>(args, stream);
     case kTile256x128: return launch_gemm_cfg<4, 1, 2, 4, true>(args, stream);
     case kTile128x128: return launch_gemm_cfg<4, 1, 1, 4, true>(args, stream);
     case kTile256x256: return launch_gemm_cfg<2, 2, 4, 4, true>(args, stream);
+    case kTile256x128w: return launch_gemm_cfg<2, 2, 4, 2, true>(args, stream);
     default: return hipErrorInvalidValue;
   }
 }
