@@ -23,6 +23,10 @@ CLOCK_HZ = 2.4e9
 DENSE_F16_PEAK_TFLOPS = CU_COUNT * CLOCK_HZ * 4096 / 1e12        # 2516.6: published dense fp16 MFMA peak
 SMFMAC_PEAK_TFLOPS = 2 * DENSE_F16_PEAK_TFLOPS                   # dense-equivalent rate of v_smfmac f16
 HBM_PEAK_GBS = 8000.0
+# HBM-side bytes per launch of the dominant kernel, from two rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE), each
+# scaled by what the same counter reads for a 256 MiB copy kernel (x2.000 and x1.000): see
+# profiles/gemm_kernel_square8192_counters.txt. Only the workload it was measured on has a figure.
+MEASURED_TRAFFIC_BYTES = {"square:8192": (356250 * 2.000 + 170470 * 1.000) * 1024}
 
 
 def parse_workload(text):
@@ -59,6 +63,30 @@ def time_launches(fn, steps, warmup):
     return start.elapsed_time(stop) / steps * 1e-3, wall / steps
 
 
+def time_graph(fn, launches, warmup=20):
+    """Average duration of one launch inside a HIP graph of `launches` back-to-back kernel nodes (no host
+    launch overhead between them). The graph is replayed once untimed and once timed."""
+    import torch
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(launches):
+                fn(i)
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    graph.replay()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / launches * 1e-3
+
+
 def run_gemm(w, steps, warmup):
     import torch
     from onebitsparsemul_amd import _native, synthetic
@@ -75,7 +103,8 @@ def run_gemm(w, steps, warmup):
 
 def run_decode_rotating(m, k, n, launches=2000, copies=None):
     """HBM-bound decode shape: rotate over enough distinct prepared weights (> 256 MiB in total, more than the
-    last-level cache) that every launch streams its weight from HBM; also time the same-buffer case."""
+    last-level cache) that every launch streams its weight from HBM; also time the same-buffer case. The
+    launches are recorded into a HIP graph so that the figure is kernel time, not host launch overhead."""
     import torch
     from onebitsparsemul_amd import _native, synthetic
     a, meta = synthetic.make_weight(m, k, seed=3, device="cuda")
@@ -87,8 +116,8 @@ def run_decode_rotating(m, k, n, launches=2000, copies=None):
     d = torch.empty((m, n), dtype=torch.float16, device="cuda")
     rot = lambda i: _native.matmul_prepared(preps[i % copies], b, d, m, n, k)
     same = lambda i: _native.matmul_prepared(prep0, b, d, m, n, k)
-    t_rot, _ = time_launches(rot, launches, 50)
-    t_same, _ = time_launches(same, launches, 50)
+    t_rot = time_graph(rot, launches)
+    t_same = time_graph(same, launches)
     nbytes = algorithmic_bytes(m, n, k, 0.0)
     return dict(shape=f"{m}x{k}x{n}", bytes=nbytes, copies=copies, launches=launches,
                 us_per_launch_hbm=t_rot * 1e6, gbps_hbm=nbytes / t_rot / 1e9,
@@ -126,6 +155,8 @@ def main():
     ap.add_argument("--workload", default="square:8192")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy kernel (reference point for HBM counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
@@ -146,6 +177,12 @@ def main():
         print(json.dumps(line))
         return
 
+    if args.calibration_copy:
+        src = torch.zeros(128 << 20, dtype=torch.float16, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
     kernel_s, wall_s, operands = run_gemm(w, args.steps, args.warmup)
     tflops = 2.0 * m * n * k / kernel_s / 1e12
     line = dict(
@@ -155,7 +192,7 @@ def main():
         config=dict(workload=w["name"], m=m, n=n, k=k, alpha=w["alpha"], beta=w["beta"], a="1-bit 2:4 prepared",
                     b="fp16 N(0,1)", accumulate="fp32", d="fp16"),
         roofline=dict(bound="mfma", achieved=tflops, peak=SMFMAC_PEAK_TFLOPS, unit="TFLOP/s",
-                      frac=tflops / SMFMAC_PEAK_TFLOPS, traffic=None,
+                      frac=tflops / SMFMAC_PEAK_TFLOPS, traffic=MEASURED_TRAFFIC_BYTES.get(w["name"]),
                       note="dense-equivalent FLOPs 2MNK against the fp16 SMFMAC rate (2 x the dense fp16 MFMA peak "
                            f"{DENSE_F16_PEAK_TFLOPS:.1f}); the same fraction as executed FLOPs MNK against the dense peak",
                       hbm_gbps_algorithmic=algorithmic_bytes(m, n, k, w["beta"]) / kernel_s / 1e9),

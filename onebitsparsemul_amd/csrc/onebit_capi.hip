@@ -79,9 +79,9 @@ int check_dtype(int c_dtype, int d_dtype) {
 int pick_tile(int m, int n) {
   const int forced = g_tile_config.load();
   if (forced >= 0) return forced;
+  // 256 x 128 workgroup tiles (two workgroups per CU) once they give every CU work; smaller tiles below that
   auto tiles = [&](int bm, int bn) { return (long)((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
-  if (tiles(512, 128) >= 256) return onebit::kTile512x128;
-  if (tiles(256, 128) >= 192) return onebit::kTile256x128;
+  if (tiles(256, 128) >= 256) return onebit::kTile256x128w;
   return onebit::kTile128x128;
 }
 
@@ -103,7 +103,7 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
     args.c_f16 = c_dtype == ONEBIT_DTYPE_F16;
     args.d_f16 = d_dtype == ONEBIT_DTYPE_F16;
     int rows = g_skinny_rows.load();
-    if (rows <= 0) rows = (m / 64 >= 256) ? 64 : 32;  // enough workgroups to cover the 256 CUs
+    if (rows <= 0) rows = (m / 64 >= 128) ? 64 : 32;  // 64-row groups once they give at least 128 workgroups
     ONEBIT_HIP(onebit::launch_skinny(args, rows, stream));
     return ONEBIT_OK;
   }
