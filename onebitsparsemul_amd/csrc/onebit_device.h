@@ -93,11 +93,24 @@ __device__ __forceinline__ half8_t expand_signs(const AChunk& a, uint32_t packed
   return __builtin_bit_cast(half8_t, v);
 }
 
-template <int STEP>
+// One SMFMAC of K step STEP. Written as inline assembly with the accumulator tied to an accumulation-register
+// tuple ("+a") and the operands to vector registers: with 256 accumulator registers in flight the compiler's own
+// allocation mixes the two register files and then copies whole accumulator tiles between them behind the SMFMAC
+// that produced them, which serialises the matrix pipe. Consecutive SMFMACs never share an accumulator, so no
+// wait states are needed between them.
+template <int STEP, bool PINNED = true>
 __device__ __forceinline__ float16_t smfmac_step(const AChunk& a, half8_t av, half16_t bv, float16_t acc) {
   const int idx = (int)a.meta[STEP / 2];
-  return __builtin_amdgcn_smfmac_f32_32x32x32_f16(av, bv, acc, idx, 0, STEP % 2);
+  // Kernels whose consecutive SMFMACs update the same accumulator use the builtin, so that the compiler inserts
+  // the wait states that dependency needs.
+  if (!PINNED) return __builtin_amdgcn_smfmac_f32_32x32x32_f16(av, bv, acc, idx, 0, STEP % 2);
+  if (STEP % 2 == 0) asm("v_smfmac_f32_32x32x32_f16 %0, %1, %2, %3" : "+a"(acc) : "v"(av), "v"(bv), "v"(idx));
+  else asm("v_smfmac_f32_32x32x32_f16 %0, %1, %2, %3 abid:1" : "+a"(acc) : "v"(av), "v"(bv), "v"(idx));
+  return acc;
 }
+
+// Wait states between the last SMFMAC and the first read of its result by a vector instruction.
+__device__ __forceinline__ void smfmac_drain() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 
 // ---- LDS transpose read ---------------------------------------------------------------------------
 // ds_read_b64_tr_b16 (measured): result element v of lane l is element l % 4 of the 8-byte chunk whose

@@ -141,8 +141,8 @@ __device__ __forceinline__ void compute_stage(const char* stage_lds, const AChun
       else av = expand_signs<2 * STAGE_IN_CHUNK + 1>(a[fm], one);
 #pragma unroll
       for (int fn = 0; fn < FN; ++fn) {
-        if (ks == 0) acc[fm][fn] = smfmac_step<2 * STAGE_IN_CHUNK>(a[fm], av, bv[fn], acc[fm][fn]);
-        else acc[fm][fn] = smfmac_step<2 * STAGE_IN_CHUNK + 1>(a[fm], av, bv[fn], acc[fm][fn]);
+        if (ks == 0) acc[fm][fn] = smfmac_step<2 * STAGE_IN_CHUNK, false>(a[fm], av, bv[fn], acc[fm][fn]);
+        else acc[fm][fn] = smfmac_step<2 * STAGE_IN_CHUNK + 1, false>(a[fm], av, bv[fn], acc[fm][fn]);
       }
     }
   }
@@ -161,6 +161,15 @@ __device__ __forceinline__ void compute_stage(const char* stage_lds, const AChun
 #endif
 #ifndef ONEBIT_EXP_COPY_MODE  /* 1: no A copies, 2: no B copies, 3: B copies never advance (always cache hits) */
 #define ONEBIT_EXP_COPY_MODE 0
+#endif
+#ifndef ONEBIT_EXP_WAIT_MODE  /* 1: never wait for copies (vmcnt 63), 2: always wait for all copies (vmcnt 0) */
+#define ONEBIT_EXP_WAIT_MODE 0
+#endif
+#ifndef ONEBIT_MAIN_PINNED   /* 1: inline-asm SMFMAC with accumulators pinned to AGPRs where that fits, 0: builtin */
+#define ONEBIT_MAIN_PINNED 1
+#endif
+#ifndef ONEBIT_MAIN_INTERLEAVE /* 1: force the order SMFMAC, LDS read, VALU inside each K-step region */
+#define ONEBIT_MAIN_INTERLEAVE 0
 #endif
 #ifndef ONEBIT_EXP_NO_BARRIER
 #define ONEBIT_EXP_NO_BARRIER 0
@@ -210,7 +219,30 @@ __device__ __forceinline__ void mfma_frags(const AChunk (&a)[FM], const half8_t 
 #pragma unroll
   for (int fm = 0; fm < FM; ++fm)
 #pragma unroll
-    for (int fn = 0; fn < FN; ++fn) acc[fm][fn] = smfmac_step<STEP>(a[fm], av[fm], bv[fn], acc[fm][fn]);
+    for (int fn = 0; fn < FN; ++fn)
+      // pinned accumulators only for the one-wavefront-per-SIMD tiles: the two-per-SIMD tiles have 128 vector
+      // registers left beside their 128 accumulators, which the pinned form overflows
+      acc[fm][fn] = smfmac_step<STEP, (ONEBIT_MAIN_PINNED != 0 && FM * FN > 8)>(a[fm], av[fm], bv[fn], acc[fm][fn]);
+}
+
+// Pins the instruction order of one K-step region: each SMFMAC is followed by its share of the region's LDS
+// reads (4 FN in total) and sign-expansion VALU instructions (8 FM in total).
+template <int FM, int FN, int I>
+__device__ __forceinline__ void interleave_from() {
+  if constexpr (I < FM * FN) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    constexpr int DS = (4 * FN * (I + 1)) / (FM * FN) - (4 * FN * I) / (FM * FN);
+    constexpr int VA = (8 * FM * (I + 1)) / (FM * FN) - (8 * FM * I) / (FM * FN);
+    if constexpr (DS > 0) __builtin_amdgcn_sched_group_barrier(0x100, DS, 0);
+    if constexpr (VA > 0) __builtin_amdgcn_sched_group_barrier(0x002, VA, 0);
+    interleave_from<FM, FN, I + 1>();
+  }
+}
+template <int FM, int FN>
+__device__ __forceinline__ void interleave_region() {
+#if ONEBIT_MAIN_INTERLEAVE
+  interleave_from<FM, FN, 0>();
+#endif
 }
 
 // Source of zeros for the asynchronous copies of B rows at or past K.
@@ -366,8 +398,9 @@ __global__ __launch_bounds__(256, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmA
       load_b_frags<FN, BN>(smem + (S) * TS::STAGE_BYTES, 1, bv1, frag_off, lane_row_off);                         \
       expand_frags<2 * (S) + 1>(a_cur, one, av1);                                                                \
       mfma_frags<2 * (S)>(a_cur, av0, bv0, acc);                                                                 \
+      interleave_region<FM, FN>();                                                                               \
       __builtin_amdgcn_sched_barrier(0); /* keep the step's work inside its region */                           \
-      wait_vmcnt_lgkm0<(WAITCNT)>(); /* copies of stage S+1 landed; this wavefront's reads of stage S returned */ \
+      wait_vmcnt_lgkm0<(ONEBIT_EXP_WAIT_MODE == 1 ? 63 : ONEBIT_EXP_WAIT_MODE == 2 ? 0 : (WAITCNT))>(); /* copies of stage S+1 landed; this wavefront's reads of stage S returned */ \
       if (!ONEBIT_EXP_NO_BARRIER) __builtin_amdgcn_s_barrier();                                                  \
       if (ISSUE_A) issue_a();                                                                                    \
       issue_b(S);                                                                                                \
@@ -379,16 +412,19 @@ __global__ __launch_bounds__(256, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmA
       ONEBIT_STAGE(0, 2 * NL, true)
       expand_frags<2>(a_cur, one, av0);
       mfma_frags<1>(a_cur, av1, bv1, acc);
+      interleave_region<FM, FN>();
       __builtin_amdgcn_sched_barrier(0);
       // mid stage 1: waits for B(4c+2); newer: B(4c+3), A(c+1), B(4c+4)
       ONEBIT_STAGE(1, 2 * NL + NA, false)
       expand_frags<4>(a_cur, one, av0);
       mfma_frags<3>(a_cur, av1, bv1, acc);
+      interleave_region<FM, FN>();
       __builtin_amdgcn_sched_barrier(0);
       // mid stage 2: waits for B(4c+3); newer: A(c+1), B(4c+4), B(4c+5)
       ONEBIT_STAGE(2, 2 * NL + NA, false)
       expand_frags<6>(a_cur, one, av0);
       mfma_frags<5>(a_cur, av1, bv1, acc);
+      interleave_region<FM, FN>();
       __builtin_amdgcn_sched_barrier(0);
       // mid stage 3: waits for B(4c+4), which is newer than A(c+1): the next chunk of A is readable after it
       ONEBIT_STAGE(3, 2 * NL, false)
@@ -401,6 +437,7 @@ __global__ __launch_bounds__(256, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmA
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) a_cur[fm] = a_next[fm];
       }
+      interleave_region<FM, FN>();
       __builtin_amdgcn_sched_barrier(0);
     }
 #undef ONEBIT_STAGE
@@ -430,6 +467,7 @@ __global__ __launch_bounds__(256, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmA
     }
   }
 
+  smfmac_drain();
   // ---- epilogue: D = alpha * acc + beta * C (csrc/kernel.h:27-31), fp16 (RNE) or fp32 output ----
   const int col_lane = lane & 31;
   const int row_lane = 4 * (lane >> 5);
@@ -549,7 +587,7 @@ __global__ __launch_bounds__(1024) void skinny_kernel(SkinnyArgs p) {
       }
       const half16_t bv = __builtin_bit_cast(half16_t, raw);
 #pragma unroll
-      for (int r = 0; r < R; ++r) acc[r] = smfmac_step<STEP>(a[r], expand_signs<STEP>(a[r], one), bv, acc[r]);
+      for (int r = 0; r < R; ++r) acc[r] = smfmac_step<STEP, false>(a[r], expand_signs<STEP>(a[r], one), bv, acc[r]);
     };
     step(std::integral_constant<int, 0>{});
     step(std::integral_constant<int, 1>{});
@@ -561,6 +599,7 @@ __global__ __launch_bounds__(1024) void skinny_kernel(SkinnyArgs p) {
     step(std::integral_constant<int, 7>{});
   }
 
+  smfmac_drain();
   // ---- add the sixteen partial tiles through LDS: region of wavefront w := its R tiles as [r][32 rows][16 cols] fp32
   {
     float* tile = reinterpret_cast<float*>(region);
@@ -635,6 +674,7 @@ hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
     case kTile128x128: return launch_gemm_cfg<4, 1, 1, 4, true>(args, stream);
     case kTile256x256: return launch_gemm_cfg<2, 2, 4, 4, true>(args, stream);
     case kTile256x128w: return launch_gemm_cfg<2, 2, 4, 2, true>(args, stream);
+    case kTile512x128t: return launch_gemm_cfg<2, 2, 8, 2, true>(args, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -650,7 +690,6 @@ hipError_t launch_skinny(SkinnyArgs args, int rows_per_group, hipStream_t stream
   switch (rows_per_group) {
     case 32: return launch_skinny_cfg<1>(args, stream);
     case 64: return launch_skinny_cfg<2>(args, stream);
-    case 128: return launch_skinny_cfg<4>(args, stream);
     default: return hipErrorInvalidValue;
   }
 }

@@ -28,12 +28,12 @@ struct SkinnyArgs {
   int c_f16, d_f16;
 };
 
-enum TileConfig { kTile512x128 = 0, kTile256x128 = 1, kTile128x128 = 2, kTile256x256 = 3, kTile256x128w = 4, kTileAuto = -1 };
+enum TileConfig { kTile512x128 = 0, kTile256x128 = 1, kTile128x128 = 2, kTile256x256 = 3, kTile256x128w = 4, kTile512x128t = 5, kTileAuto = -1 };
 
 hipError_t launch_prepare(const void* a, const void* e, void* prep, int m, int k, int layout, hipStream_t stream);
 hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream);
 
-// Split-K kernel for n <= 16; rows_per_group (32, 64 or 128) = weight rows one workgroup covers.
+// Split-K kernel for n <= 16; rows_per_group (32 or 64) = weight rows one workgroup covers.
 constexpr int kSkinnyMaxN = 16;
 hipError_t launch_skinny(SkinnyArgs args, int rows_per_group, hipStream_t stream);
 
