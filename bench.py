@@ -155,6 +155,7 @@ def main():
     ap.add_argument("--workload", default="square:8192")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--no-ceiling", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy kernel (reference point for HBM counters)")
     args = ap.parse_args()
@@ -197,6 +198,13 @@ def main():
                            f"{DENSE_F16_PEAK_TFLOPS:.1f}); the same fraction as executed FLOPs MNK against the dense peak",
                       hbm_gbps_algorithmic=algorithmic_bytes(m, n, k, w["beta"]) / kernel_s / 1e9),
         wall_ms_per_step=wall_s * 1e3)
+    if not args.no_ceiling:
+        # register-only SMFMAC loops: what the chip sustains under matrix load, which depends on the operand values
+        from onebitsparsemul_amd import _native
+        line["smfmac_register_loop_tflops"] = dict(
+            benchmark_distribution=max(_native.measure_smfmac_rate(True, 50000) for _ in range(2)),
+            constant_operands=max(_native.measure_smfmac_rate(False, 50000) for _ in range(2)),
+            note="no LDS or global memory in the loop; the gap to the nominal peak is clock throttling under load")
     if not args.no_decode:
         line["decode_n16"] = run_decode_rotating(11008, 4096, 16)
     if not args.no_cpu_baseline:

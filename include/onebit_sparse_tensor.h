@@ -74,6 +74,15 @@ int onebit_sparse_prepare(const void *a, const void *e, int m, int k, int meta_l
 int onebit_sparse_matmul_prepared(const void *prepared, const void *b, const void *c, void *d, int m, int n, int k,
                                   float alpha, float beta, int c_dtype, int d_dtype, void *stream);
 
+/*
+ * Packs a dense fp16 weight (m x k, row-major, device) into the stored operands a (m*k/16 bytes) and e
+ * (m*k/8 bytes) on the GPU. Replaces the tensor-op pipeline of BinaryLinear_2_4.pack
+ * (onebit_sparse_mul/__init__.py:130-145 with _semi_structured_conversions.py:54-179,286-314): prune != 0 first
+ * keeps the two largest magnitudes of every aligned group of four (among equal magnitudes the lower index is
+ * pruned), prune == 0 takes the weight's non-zero pattern as it is.
+ */
+int onebit_sparse_pack(const void *weight, int m, int k, int prune, void *a, void *e, int meta_layout, void *stream);
+
 /* Message of the last failure on the calling thread ("" if none). Host pointer, valid until the next call. */
 const char *onebit_sparse_last_error(void);
 
@@ -83,6 +92,13 @@ void onebit_sparse_set_tile_config(int tile_config);
 void onebit_sparse_set_skinny_enabled(int enabled);
 /* Weight rows one workgroup of the split-K kernel covers: 32 or 64; <= 0 = automatic. */
 void onebit_sparse_set_skinny_rows(int rows);
+
+/* Diagnostic, no counterpart in the reference: sustained rate of v_smfmac_f32_32x32x32_f16 in a register-only
+ * loop on the current device (one wavefront per SIMD, `iterations` x 16 instructions each), in dense-equivalent
+ * TFLOP/s. random_operands = 1 uses +-1 values, N(0,1) fp16 B values and random 2:4 indices (the benchmark's
+ * distribution), 0 uses constants. The clock the GPU sustains under matrix load depends on the operand values, so
+ * this is the practical ceiling next to the nominal peak. Allocates and frees its own device buffers; synchronous. */
+int onebit_sparse_measure_smfmac_rate(int random_operands, int iterations, double *dense_equiv_tflops);
 
 #ifdef __cplusplus
 }

@@ -132,6 +132,12 @@ class BinaryLinear_2_4(nn.Module):
         Reference: onebit_sparse_mul/__init__.py:130-145."""
         if tuple(weight.shape) != (self.outfeatures, self.infeatures):
             raise ValueError(f"weight must have shape ({self.outfeatures}, {self.infeatures})")
+        if weight.is_cuda and weight.dtype == torch.float16:
+            # one fused HIP kernel (mask, compress, quantise, transpose-pack, reorder); same result as below
+            self.packed_binary_sparse, self.meta = _native.pack_weight(weight.contiguous(), prune=True)
+            self.vaild = True
+            self._prepared = None
+            return
         w = weight * mask_creator(weight).to(weight.dtype)
         if w.dtype not in (torch.half, torch.bfloat16, torch.int32):
             w = w.to(torch.half)

@@ -14,8 +14,8 @@ META_REFERENCE, META_CUTLASS, META_LOGICAL = 0, 1, 2
 
 EXPORTS = (
     "onebit_sparse_matmul", "onebit_sparse_matmul_ex", "onebit_sparse_prepared_bytes", "onebit_sparse_prepare",
-    "onebit_sparse_matmul_prepared", "onebit_sparse_last_error", "onebit_sparse_set_tile_config",
-    "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows",
+    "onebit_sparse_matmul_prepared", "onebit_sparse_pack", "onebit_sparse_last_error", "onebit_sparse_set_tile_config",
+    "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_measure_smfmac_rate",
 )
 
 _lib = None
@@ -38,6 +38,8 @@ def lib():
         L.onebit_sparse_prepare.argtypes = [vp, vp, i32, i32, i32, vp, vp]
         L.onebit_sparse_matmul_prepared.restype = i32
         L.onebit_sparse_matmul_prepared.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, i32, vp]
+        L.onebit_sparse_pack.restype = i32
+        L.onebit_sparse_pack.argtypes = [vp, i32, i32, i32, vp, vp, i32, vp]
         L.onebit_sparse_last_error.restype = ctypes.c_char_p
         L.onebit_sparse_last_error.argtypes = []
         L.onebit_sparse_set_tile_config.restype = None
@@ -46,6 +48,8 @@ def lib():
         L.onebit_sparse_set_skinny_enabled.argtypes = [i32]
         L.onebit_sparse_set_skinny_rows.restype = None
         L.onebit_sparse_set_skinny_rows.argtypes = [i32]
+        L.onebit_sparse_measure_smfmac_rate.restype = i32
+        L.onebit_sparse_measure_smfmac_rate.argtypes = [i32, i32, ctypes.POINTER(ctypes.c_double)]
         _lib = L
     return _lib
 
@@ -145,3 +149,26 @@ def set_skinny_enabled(flag):
 
 def set_skinny_rows(rows):
     lib().onebit_sparse_set_skinny_rows(rows)
+
+
+def measure_smfmac_rate(random_operands=True, iterations=50000):
+    """Sustained register-only SMFMAC rate of the current GPU, dense-equivalent TFLOP/s (diagnostic)."""
+    out = ctypes.c_double(0.0)
+    rc = lib().onebit_sparse_measure_smfmac_rate(1 if random_operands else 0, iterations, ctypes.byref(out))
+    if rc != 0:
+        raise RuntimeError(f"libonebitmul: measuring the SMFMAC rate failed (status {rc})")
+    return out.value
+
+
+def pack_weight(weight, prune=True, layout=META_REFERENCE):
+    """dense fp16 (m, k) on the GPU -> (a uint8 (k/2, m/8), meta int16 (m, k/16)), the stored operands."""
+    dev = _require_cuda(weight)
+    if weight.dtype != torch.float16 or weight.dim() != 2:
+        raise TypeError("weight must be a 2-dimensional float16 tensor")
+    m, k = weight.shape
+    a = torch.empty((k // 2, m // 8), dtype=torch.uint8, device=dev)
+    meta = torch.empty((m, k // 16), dtype=torch.int16, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib().onebit_sparse_pack(weight.data_ptr(), m, k, 1 if prune else 0, a.data_ptr(), meta.data_ptr(), layout,
+                                        _stream(weight)))
+    return a, meta

@@ -27,7 +27,7 @@ def _run(cmd):
 
 def build_library():
     objs = []
-    for src in ("onebit_kernels.hip", "onebit_capi.hip"):
+    for src in ("onebit_kernels.hip", "onebit_capi.hip", "onebit_diag.hip"):
         obj = os.path.join(CSRC, src.replace(".hip", ".o"))
         _run([HIPCC, *HIP_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj])
         objs.append(obj)

@@ -147,6 +147,20 @@ int onebit_sparse_prepare(const void* a, const void* e, int m, int k, int meta_l
   return ONEBIT_OK;
 }
 
+int onebit_sparse_pack(const void* weight, int m, int k, int prune, void* a, void* e, int meta_layout, void* stream) {
+  g_last_error.clear();
+  if (int rc = check_shape(m, 1, k)) return rc;
+  if (!weight || !a || !e) return fail(ONEBIT_ERR_ARGUMENT, "null operand pointer");
+  if ((reinterpret_cast<uintptr_t>(weight) & 15) != 0)
+    return fail(ONEBIT_ERR_ARGUMENT, "the dense weight must be 16-byte aligned");
+  if ((reinterpret_cast<uintptr_t>(a) & 7) != 0 || (reinterpret_cast<uintptr_t>(e) & 1) != 0)
+    return fail(ONEBIT_ERR_ARGUMENT, "a must be 8-byte aligned and e 2-byte aligned");
+  if (meta_layout < ONEBIT_META_REFERENCE || meta_layout > ONEBIT_META_LOGICAL)
+    return fail(ONEBIT_ERR_ARGUMENT, "unknown metadata layout %d", meta_layout);
+  ONEBIT_HIP(onebit::launch_pack(weight, a, e, m, k, prune, meta_layout, static_cast<hipStream_t>(stream)));
+  return ONEBIT_OK;
+}
+
 int onebit_sparse_matmul_prepared(const void* prepared, const void* b, const void* c, void* d, int m, int n, int k,
                                   float alpha, float beta, int c_dtype, int d_dtype, void* stream) {
   g_last_error.clear();

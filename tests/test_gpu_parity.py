@@ -343,3 +343,42 @@ def test_linear_layer_forward_matches_host_check():
     # N(0,1) activations, 3-D input
     got3 = layer(x3.cuda()).cpu().double()
     assert (got3 - want3).abs().max() <= REL_TOL * want3.abs().max()
+
+
+def test_benchmark_cli_reference_check():
+    """The a.out-style benchmark (reference flags) with its reference check switched on."""
+    from onebitsparsemul_amd import benchmark
+    assert benchmark.main(["--a_rows=512", "--n=256", "--a_cols=512", "--reference-check=true", "--iterations=2"]) == 0
+    assert benchmark.main(["--a_rows=1024", "--n=16", "--a_cols=512", "--alpha=0.5", "--beta=1", "--reference-check=true",
+                           "--iterations=2", "--fp16-out"]) == 0
+
+
+@pytest.mark.parametrize("prune", [True, False])
+def test_gpu_packer_matches_host_pipeline(prune):
+    """onebit_sparse_pack (fused HIP kernel) against the oracle's mask + compress + quantise + pack, ties included."""
+    rng = np.random.default_rng(31 + prune)
+    m, k = 256, 192
+    if prune:
+        w = rng.integers(-3, 4, size=(m, k)).astype(np.float32)       # many equal magnitudes and zeros
+        w[:64] = rng.standard_normal((64, k)).astype(np.float16).astype(np.float32)
+        masked = w * oracle.mask_creator(w)
+    else:
+        masked = np.zeros((m, k // 4, 4), dtype=np.float32)            # every non-zero pattern, 0..4 per group
+        flags = rng.integers(0, 2, size=masked.shape).astype(bool)
+        masked[flags] = rng.choice([-2.0, -1.0, 1.0, 3.0], size=int(flags.sum()))
+        masked = masked.reshape(m, k)
+        w = masked
+    sparse, meta_want = oracle.sparse_from_dense(masked)
+    a_want = oracle.pack_binary(np.ascontiguousarray(oracle.binary_quant(sparse).T))
+    a, meta = _native.pack_weight(torch.from_numpy(w).half().cuda(), prune=prune)
+    torch.cuda.synchronize()
+    assert np.array_equal(meta.cpu().numpy(), meta_want)
+    assert np.array_equal(a.cpu().numpy(), a_want)
+    # and through the module: packing on the GPU equals packing on the host
+    if prune:
+        layer_gpu = ob.BinaryLinear_2_4(k, m).cuda()
+        layer_gpu.pack(torch.from_numpy(w).half().cuda())
+        layer_cpu = ob.BinaryLinear_2_4(k, m)
+        layer_cpu.pack(torch.from_numpy(w).half())
+        assert torch.equal(layer_gpu.meta.cpu(), layer_cpu.meta)
+        assert torch.equal(layer_gpu.packed_binary_sparse.cpu(), layer_cpu.packed_binary_sparse)
