@@ -602,6 +602,7 @@ __global__ __launch_bounds__(1024) void skinny_kernel(SkinnyArgs p) {
   // lanes 16-31 and 48-63 would hold columns 16-31: they re-read columns 0-15 and are never stored
   const char* lane_ptr = region + (8 * gb + (i16 >> 2)) * 32 + (i16 & 3) * 8;
   const bool vector_b = p.n == 16 && (reinterpret_cast<uintptr_t>(p.b) & 15) == 0;
+  const bool vector8_b = (p.n == 4 || p.n == 8) && (reinterpret_cast<uintptr_t>(p.b) & 15) == 0;
 
   for (int kc = wave; kc < p.kc_total; kc += kSkinnyWaves) {
     AChunk a[R];
@@ -626,6 +627,27 @@ __global__ __launch_bounds__(1024) void skinny_kernel(SkinnyArgs p) {
       }
 #pragma unroll
       for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4_t*>(region + (lane + i * 64) * 16) = v[i];
+    } else if (vector8_b) {
+      // n == 4 (or n == 8): a row is 8 (16) bytes; four rows per lane, padded to the 32-byte LDS rows
+#pragma unroll
+      for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4_t*>(region + (lane + i * 64) * 16) = u32x4_t{0, 0, 0, 0};
+      const int row_bytes = p.n * 2;
+      const char* src = reinterpret_cast<const char*>(p.b) + (size_t)k_base * row_bytes;
+      u32x4_t v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = lane + i * 64;
+        const char* q = src + (size_t)(row < rows_valid ? row : 0) * row_bytes;
+        if (p.n == 4) {
+          const u32x2_t t = *reinterpret_cast<const u32x2_t*>(q);
+          v[i] = u32x4_t{t.x, t.y, 0, 0};
+        } else {
+          v[i] = *reinterpret_cast<const u32x4_t*>(q);
+        }
+        if (row >= rows_valid) v[i] = u32x4_t{0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4_t*>(region + (lane + i * 64) * 32) = v[i];
     } else {
       // any n <= 16, any alignment: the valid part of the chunk is one run of rows_valid * n elements
 #pragma unroll
