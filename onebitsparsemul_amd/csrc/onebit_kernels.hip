@@ -169,22 +169,25 @@ struct TileShape {
   static_assert(NL >= 1, "tile too narrow for the copy pattern");
 };
 
-// XCD-aware tile order: workgroup b runs on XCD b % 8, so XCD x is given a contiguous range of the tile
-// list, and the list itself walks tiles in groups of eight row tiles so that the ~32 tiles resident on
-// one XCD share A row panels and B column panels in that XCD's L2.
+// XCD-aware tile order. Workgroup b runs on XCD b % 8, so XCD x is given a contiguous range of a tile list
+// that is ordered in blocks of 16 row tiles x 4 column tiles (row tile fastest), blocks running down M inside a
+// strip of 4 column tiles, strips running along N. The ~64 workgroups resident on one XCD then form one block:
+// every B column panel it streams is shared by 16 workgroups and every A row panel by 4 in that XCD's L2, and
+// the whole range of one XCD covers few column strips, so B is fetched into few L2s.
 __device__ __forceinline__ void tile_of_block(int b, int tiles_m, int tiles_n, int& tm, int& tn) {
   const int total = tiles_m * tiles_n;
   const int per = total / 8, rem = total % 8;
   const int x = b % 8, local = b / 8;
   const int v = x * per + (x < rem ? x : rem) + local;
-  constexpr int GROUP_M = 8;
-  const int in_group = GROUP_M * tiles_n;
-  const int g = v / in_group;
-  const int first_m = g * GROUP_M;
-  const int gsz = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
-  const int w = v % in_group;
-  tm = first_m + w % gsz;
-  tn = w / gsz;
+  constexpr int GROUP_M = 16, STRIP_N = 4;
+  const int strip = v / (tiles_m * STRIP_N);
+  const int strip_w = (tiles_n - strip * STRIP_N) < STRIP_N ? (tiles_n - strip * STRIP_N) : STRIP_N;
+  const int w = v - strip * STRIP_N * tiles_m;
+  const int group = w / (GROUP_M * strip_w);
+  const int group_h = (tiles_m - group * GROUP_M) < GROUP_M ? (tiles_m - group * GROUP_M) : GROUP_M;
+  const int u = w - group * GROUP_M * strip_w;
+  tm = group * GROUP_M + u % group_h;
+  tn = strip * STRIP_N + u / group_h;
 }
 
 // One stage (64 K = two SMFMAC K steps) of a wavefront's FM x FN tile.
@@ -193,8 +196,6 @@ __device__ __forceinline__ void compute_stage(const char* stage_lds, const AChun
                                               const int (&frag_off)[FN], int lane_row_off, uint32_t one) {
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks) {
-    constexpr int dummy = 0;
-    (void)dummy;
     half16_t bv[FN];
 #pragma unroll
     for (int fn = 0; fn < FN; ++fn) {
