@@ -778,6 +778,8 @@ hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
     case kTile256x256: return launch_gemm_cfg<2, 2, 4, 4, true>(args, stream);
     case kTile256x128w: return launch_gemm_cfg<2, 2, 4, 2, true>(args, stream);
     case kTile512x128t: return launch_gemm_cfg<2, 2, 8, 2, true>(args, stream);
+    case kTile128x128s: return launch_gemm_cfg<2, 2, 2, 2, true>(args, stream);
+    case kTile256x64: return launch_gemm_cfg<2, 2, 4, 1, true>(args, stream);
     default: return hipErrorInvalidValue;
   }
 }
