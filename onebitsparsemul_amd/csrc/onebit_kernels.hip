@@ -672,19 +672,25 @@ __global__ __launch_bounds__(1024) void skinny_kernel(SkinnyArgs p) {
     }
     // the region is private to this wavefront and its LDS operations execute in order: no barrier needed
 
-    auto step = [&](auto step_tag) {
-      constexpr int STEP = decltype(step_tag)::value;
+    // all B fragments of the chunk first (32 transpose reads in flight), then the SMFMACs back to back
+    half16_t bfrag[kStepsPerChunk];
+#pragma unroll
+    for (int st = 0; st < kStepsPerChunk; ++st) {
       u32x8_t raw;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int row_const = STEP * 32 + 4 * (q & 1) + 16 * (q >> 1);
+        const int row_const = st * 32 + 4 * (q & 1) + 16 * (q >> 1);
         const u32x2_t t = lds_read_tr16(lane_ptr + row_const * 32);
         raw[2 * q] = t.x;
         raw[2 * q + 1] = t.y;
       }
-      const half16_t bv = __builtin_bit_cast(half16_t, raw);
+      bfrag[st] = __builtin_bit_cast(half16_t, raw);
+    }
+    auto step = [&](auto step_tag) {
+      constexpr int STEP = decltype(step_tag)::value;
 #pragma unroll
-      for (int r = 0; r < R; ++r) acc[r] = smfmac_step<STEP, false>(a[r], expand_signs<STEP>(a[r], one), bv, acc[r]);
+      for (int r = 0; r < R; ++r)
+        acc[r] = smfmac_step<STEP, false>(a[r], expand_signs<STEP>(a[r], one), bfrag[STEP], acc[r]);
     };
     step(std::integral_constant<int, 0>{});
     step(std::integral_constant<int, 1>{});
@@ -756,12 +762,16 @@ static hipError_t launch_gemm_cfg(GemmArgs args, hipStream_t stream) {
   args.tiles_n = (args.n + TS::BN - 1) / TS::BN;
   const int lds = DMA ? TS::LDS_BYTES : TS::STAGE_BYTES;
   auto kern = gemm_kernel<WM, WN, FM, FN, DMA>;
-  static bool attr_done = false;  // per instantiation; racing writers store the same value
-  if (!attr_done) {
+  // the dynamic-LDS limit is a per-device attribute of the kernel; racing writers store the same value
+  static bool attr_done[64] = {};
+  int device = 0;
+  if (hipError_t st = hipGetDevice(&device); st != hipSuccess) return st;
+  if (device < 0 || device >= 64) return hipErrorInvalidDevice;
+  if (!attr_done[device]) {
     hipError_t st = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (st != hipSuccess) return st;
-    attr_done = true;
+    attr_done[device] = true;
   }
   hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n), dim3(256), lds, stream, args);
   return hipGetLastError();

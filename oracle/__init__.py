@@ -177,10 +177,10 @@ def blas_matmul(a_dense, b_half, c=None, alpha=1.0, beta=0.0, dtype=np.float64):
     return out
 
 
-def cpu_baseline_gemm(a, b_half, e, m, n, k, row_begin, row_end, layout=LAYOUT_REFERENCE, threads=None):
+def cpu_baseline_gemm(a, b_half, e, m, n, k, row_begin, row_end, layout=LAYOUT_REFERENCE, threads=None, repeats=1):
     """The reference's CPU path (onebit_sparse_mul/__init__.py:67-97: decompress the weight, then a dense
-    torch.matmul) on rows [row_begin, row_end) of A, in fp32 on the host's cores. Returns (seconds of the
-    matmul, seconds of the decompression, result slab as float32 numpy)."""
+    torch.matmul) on rows [row_begin, row_end) of A, in fp32 on the host's cores. Returns (seconds of one
+    matmul, averaged over `repeats`; seconds of the decompression; result slab as float32 numpy)."""
     import time
 
     import torch
@@ -194,6 +194,7 @@ def cpu_baseline_gemm(a, b_half, e, m, n, k, row_begin, row_end, layout=LAYOUT_R
     b_t = torch.from_numpy(np.ascontiguousarray(b_half)).to(torch.float32)
     torch.matmul(a_t[:64], b_t)  # warm-up of the BLAS threads
     t2 = time.perf_counter()
-    out = torch.matmul(a_t, b_t)
+    for _ in range(repeats):
+        out = torch.matmul(a_t, b_t)
     t3 = time.perf_counter()
-    return t3 - t2, t1 - t0, out.numpy()
+    return (t3 - t2) / repeats, t1 - t0, out.numpy()
