@@ -141,7 +141,7 @@ __global__ __launch_bounds__(64) void pack_kernel(const _Float16* __restrict__ w
 
 // =====================================================================================================
 // Main kernel.
-// Workgroup = 4 wavefronts arranged WM x WN; each wavefront owns FM x FN accumulator tiles of 32 x 32.
+// Workgroup = 4 or 8 wavefronts arranged WM x WN; each wavefront owns FM x FN accumulator tiles of 32 x 32.
 // B is staged through LDS in stages of 64 K rows; the LDS image of a stage is row-major (N contiguous)
 // with the 16-byte column chunks of row r XOR-swizzled so that the four rows a 16-lane group touches in
 // one transpose read fall into different bank groups.
@@ -160,12 +160,14 @@ struct TileShape {
   static constexpr int BM = WM * FM * 32;
   static constexpr int BN = WN * FN * 32;
   static constexpr int CH = BN / 8;                       // 16-byte chunks per LDS row
-  static constexpr int NL = kStageK * CH / 256;           // chunk copies per thread per stage
+  static constexpr int NW = WM * WN;                      // wavefronts per workgroup
+  static constexpr int NL = kStageK * CH / (64 * NW);     // chunk copies per thread per stage
   static constexpr int STAGE_BYTES = kStageK * BN * 2;
   static constexpr int LDS_B_BYTES = kStages * STAGE_BYTES;
-  static constexpr int NA = ((BM / 32) * 1536 + 4095) / 4096;  // 1 KiB A copies per wavefront per K chunk
-  static constexpr int LDS_BYTES = LDS_B_BYTES + NA * 4096;
-  static_assert(WM * WN == 4, "four wavefronts per workgroup");
+  static constexpr int NA = ((BM / 32) * 1536 + 1024 * NW - 1) / (1024 * NW);  // 1 KiB A copies per wavefront per chunk
+  static constexpr int LDS_BYTES = LDS_B_BYTES + NA * 1024 * NW;
+  static_assert(NW == 4 || NW == 8, "four or eight wavefronts per workgroup");
+  static_assert(kStageK * CH % (64 * NW) == 0, "the stage must divide into whole wavefront copies");
   static_assert(NL >= 1, "tile too narrow for the copy pattern");
 };
 
@@ -234,7 +236,8 @@ __device__ __forceinline__ void compute_stage(const char* stage_lds, const AChun
 #ifndef ONEBIT_EXP_NO_COPY
 #define ONEBIT_EXP_NO_COPY 0
 #endif
-#ifndef ONEBIT_EXP_COPY_MODE  /* 1: no A copies, 2: no B copies, 3: B copies never advance (always cache hits) */
+#ifndef ONEBIT_EXP_COPY_MODE  /* 1: no A copies, 2: no B copies, 3: B copies never advance (always cache hits),
+                                 5: only every other B copy (half the L2->LDS traffic, same addresses otherwise) */
 #define ONEBIT_EXP_COPY_MODE 0
 #endif
 #ifndef ONEBIT_EXP_WAIT_MODE  /* 1: never wait for copies (vmcnt 63), 2: always wait for all copies (vmcnt 0) */
@@ -324,9 +327,9 @@ __device__ __forceinline__ void interleave_region() {
 __device__ __attribute__((aligned(16))) uint32_t g_zero16[4] = {0, 0, 0, 0};
 
 template <int WM, int WN, int FM, int FN, bool DMA>
-__global__ __launch_bounds__(256, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmArgs p) {
+__global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmArgs p) {
   using TS = TileShape<WM, WN, FM, FN>;
-  constexpr int BM = TS::BM, BN = TS::BN, CH = TS::CH, NL = TS::NL;
+  constexpr int BM = TS::BM, BN = TS::BN, CH = TS::CH, NL = TS::NL, NW = TS::NW;
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -375,7 +378,7 @@ __global__ __launch_bounds__(256, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmA
 
   if constexpr (DMA) {
     // ---- asynchronous copy pattern for B: NL 16-byte copies per thread per stage ----
-    // copy i of wavefront w fills LDS slots [(4 i + w) * 64, +64) of the stage; slot = (row, physical chunk).
+    // copy i of wavefront w fills LDS slots [(NW i + w) * 64, +64) of the stage; slot = (row, physical chunk).
     // Global address = wave-uniform base of the stage + per-lane byte offset.
     uint32_t b_off[NL];
     int copy_row[NL];
@@ -383,14 +386,14 @@ __global__ __launch_bounds__(256, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmA
     const uint32_t smem_base = lds_offset_of(smem);
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-      const int slot = (4 * i + wave) * 64 + lane;
+      const int slot = (NW * i + wave) * 64 + lane;
       const int row = slot / CH, pc = slot % CH;
       const int lc = pc ^ chunk_swizzle<BN>(row);
       int col = 8 * lc;
       if (n0 + col >= p.n) col = 0;  // columns past N: any valid address will do, the results are not stored
       b_off[i] = (uint32_t)(row * p.n + col) * 2u;
       copy_row[i] = row;
-      lds_dst[i] = smem_base + (4 * i + wave) * 1024;
+      lds_dst[i] = smem_base + (NW * i + wave) * 1024;
     }
     const char* b_stage = reinterpret_cast<const char*>(p.b) + (size_t)n0 * 2;  // advances one stage per copy
     const size_t stage_stride = (size_t)kStageK * p.n * 2;
@@ -403,7 +406,9 @@ __global__ __launch_bounds__(256, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmA
       if (ONEBIT_EXP_NO_COPY || ONEBIT_EXP_COPY_MODE == 2) return;
       if (next_k0 + kStageK <= p.k) {  // wave-uniform: a full stage
 #pragma unroll
-        for (int i = 0; i < NL; ++i) lds_dma16_base(b_stage, b_off[i], lds_dst[i] + ring * TS::STAGE_BYTES);
+        for (int i = 0; i < NL; ++i)
+          if (ONEBIT_EXP_COPY_MODE != 5 || (i & 1) == 0)
+            lds_dma16_base(b_stage, b_off[i], lds_dst[i] + ring * TS::STAGE_BYTES);
       } else {
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
@@ -426,13 +431,13 @@ __global__ __launch_bounds__(256, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmA
       const int rb0 = tile_m * (BM / kRowBlock);
 #pragma unroll
       for (int j = 0; j < NA; ++j) {
-        const int byte = (4 * j + wave) * 1024 + lane * 16;
+        const int byte = (NW * j + wave) * 1024 + lane * 16;
         int blk = byte / kBlockBytes, off = byte % kBlockBytes;
         if (blk >= BM / kRowBlock) blk = 0;
         int rb = rb0 + blk;
         if (rb >= rb_total) rb = rb_total - 1;
         a_off[j] = (uint32_t)((size_t)rb * p.kc_total * kBlockBytes + off);  // the launcher checks it fits 32 bits
-        a_dst[j] = smem_base + TS::LDS_B_BYTES + (4 * j + wave) * 1024;
+        a_dst[j] = smem_base + TS::LDS_B_BYTES + (NW * j + wave) * 1024;
       }
     }
     const char* a_chunk = reinterpret_cast<const char*>(p.prep);  // advances one K chunk per copy
@@ -526,7 +531,7 @@ __global__ __launch_bounds__(256, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmA
       auto fill = [&](int stage) {
         const int k0 = (kc * kStages + stage) * kStageK;
         __syncthreads();
-        for (int idx = tid; idx < kStageK * BN; idx += 256) {
+        for (int idx = tid; idx < kStageK * BN; idx += 64 * NW) {
           const int row = idx / BN, col = idx % BN;
           _Float16 v = (_Float16)0.f;
           if (k0 + row < p.k && n0 + col < p.n) v = p.b[(size_t)(k0 + row) * p.n + n0 + col];
@@ -773,7 +778,7 @@ static hipError_t launch_gemm_cfg(GemmArgs args, hipStream_t stream) {
     if (st != hipSuccess) return st;
     attr_done[device] = true;
   }
-  hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n), dim3(256), lds, stream, args);
+  hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n), dim3(64 * TS::NW), lds, stream, args);
   return hipGetLastError();
 }
 
@@ -790,6 +795,8 @@ hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
     case kTile512x128t: return launch_gemm_cfg<2, 2, 8, 2, true>(args, stream);
     case kTile128x128s: return launch_gemm_cfg<2, 2, 2, 2, true>(args, stream);
     case kTile256x64: return launch_gemm_cfg<2, 2, 4, 1, true>(args, stream);
+    case kTile256x256w8: return launch_gemm_cfg<2, 4, 4, 2, true>(args, stream);
+    case kTile512x128w8: return launch_gemm_cfg<4, 2, 4, 2, true>(args, stream);
     default: return hipErrorInvalidValue;
   }
 }
