@@ -549,6 +549,90 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
 
   smfmac_drain();
   // ---- epilogue: D = alpha * acc + beta * C (csrc/kernel.h:27-31), fp16 (RNE) or fp32 output ----
+  if constexpr (DMA) {
+    if (p.vector_epilogue) {
+      // Coalesced form: each wavefront turns one 32-row block of its tile at a time through a private LDS
+      // scratch (fp32, row-major) so that every lane then handles 16 bytes of one output row: C is read and D
+      // written in full 128-byte segments instead of 64-byte (fp16) pieces per accumulator register.
+      __syncthreads();  // every wavefront is done with the stage ring, which becomes the scratch
+      constexpr int WCOLS = FN * 32;                   // columns of the wavefront's tile
+      float* scratch = reinterpret_cast<float*>(smem) + wave * (32 * WCOLS);
+      const int col_lane = lane & 31, row_lane = 4 * (lane >> 5);
+#pragma unroll
+      for (int fm = 0; fm < FM; ++fm) {
+#pragma unroll
+        for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+          for (int v = 0; v < 16; ++v)
+            scratch[(8 * (v / 4) + row_lane + (v % 4)) * WCOLS + fn * 32 + col_lane] = acc[fm][fn][v];
+        const int row_base = row0 + fm * 32;
+        if (p.d_f16) {
+          constexpr int PER_ROW = WCOLS / 8;           // 16-byte pieces (8 halves) per row
+#pragma unroll
+          for (int it = 0; it < 32 * PER_ROW / 64; ++it) {
+            const int piece = it * 64 + lane;
+            const int r = piece / PER_ROW, c8 = (piece % PER_ROW) * 8;
+            const int row = row_base + r, col = col0 + c8;
+            const float4 lo = *reinterpret_cast<const float4*>(scratch + r * WCOLS + c8);
+            const float4 hi = *reinterpret_cast<const float4*>(scratch + r * WCOLS + c8 + 4);
+            float x[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            if (row < p.m && col < p.n && !(ONEBIT_EXP_NO_STORE && x[0] != 12345.f)) {
+              const size_t o = (size_t)row * p.n + col;
+#pragma unroll
+              for (int j = 0; j < 8; ++j) x[j] = p.alpha * x[j];
+              if (p.beta != 0.f) {
+                if (p.c_f16) {
+                  const half8_t cv = *reinterpret_cast<const half8_t*>(reinterpret_cast<const _Float16*>(p.c) + o);
+#pragma unroll
+                  for (int j = 0; j < 8; ++j) x[j] = x[j] + p.beta * (float)cv[j];
+                } else {
+                  const float4 c0 = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.c) + o);
+                  const float4 c1 = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.c) + o + 4);
+                  const float cv[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+#pragma unroll
+                  for (int j = 0; j < 8; ++j) x[j] = x[j] + p.beta * cv[j];
+                }
+              }
+              half8_t out;
+#pragma unroll
+              for (int j = 0; j < 8; ++j) out[j] = (_Float16)x[j];
+              *reinterpret_cast<half8_t*>(reinterpret_cast<_Float16*>(p.d) + o) = out;
+            }
+          }
+        } else {
+          constexpr int PER_ROW = WCOLS / 4;           // 16-byte pieces (4 floats) per row
+#pragma unroll
+          for (int it = 0; it < 32 * PER_ROW / 64; ++it) {
+            const int piece = it * 64 + lane;
+            const int r = piece / PER_ROW, c4 = (piece % PER_ROW) * 4;
+            const int row = row_base + r, col = col0 + c4;
+            const float4 a4 = *reinterpret_cast<const float4*>(scratch + r * WCOLS + c4);
+            float x[4] = {a4.x, a4.y, a4.z, a4.w};
+            if (row < p.m && col < p.n && !(ONEBIT_EXP_NO_STORE && x[0] != 12345.f)) {
+              const size_t o = (size_t)row * p.n + col;
+#pragma unroll
+              for (int j = 0; j < 4; ++j) x[j] = p.alpha * x[j];
+              if (p.beta != 0.f) {
+                if (p.c_f16) {
+                  const _Float16* cp = reinterpret_cast<const _Float16*>(p.c) + o;
+#pragma unroll
+                  for (int j = 0; j < 4; ++j) x[j] = x[j] + p.beta * (float)cp[j];
+                } else {
+                  const float4 c0 = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.c) + o);
+                  const float cv[4] = {c0.x, c0.y, c0.z, c0.w};
+#pragma unroll
+                  for (int j = 0; j < 4; ++j) x[j] = x[j] + p.beta * cv[j];
+                }
+              }
+              *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.d) + o) = float4{x[0], x[1], x[2], x[3]};
+            }
+          }
+        }
+      }
+      return;
+    }
+  }
+  // Direct form (generic variant, or C / D not 16-byte aligned): one element per accumulator register.
   const int col_lane = lane & 31;
   const int row_lane = 4 * (lane >> 5);
 #pragma unroll
@@ -785,6 +869,9 @@ static hipError_t launch_gemm_cfg(GemmArgs args, hipStream_t stream) {
 hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
   if (prepared_bytes(args.m, args.k) >= (size_t(1) << 32)) return hipErrorInvalidValue;  // 32-bit copy offsets
   const bool aligned = (args.n % 8 == 0) && ((reinterpret_cast<uintptr_t>(args.b) & 15) == 0);
+  // the coalesced epilogue moves 16 bytes per lane: n % 8 == 0 keeps every row start aligned when the bases are
+  args.vector_epilogue = (reinterpret_cast<uintptr_t>(args.d) & 15) == 0 &&
+                         (args.beta == 0.f || (reinterpret_cast<uintptr_t>(args.c) & 15) == 0);
   if (!aligned) return launch_gemm_cfg<4, 1, 1, 4, false>(args, stream);
   switch (tile_config) {
     case kTile512x128: return launch_gemm_cfg<4, 1, 4, 4, true>(args, stream);

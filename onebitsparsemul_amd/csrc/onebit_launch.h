@@ -15,6 +15,7 @@ struct GemmArgs {
   float alpha, beta;
   int c_f16, d_f16;      // 1: fp16, 0: fp32
   int tiles_m, tiles_n;  // filled by the launcher
+  int vector_epilogue;   // filled by the launcher: C and D allow 16-byte accesses
 };
 
 struct SkinnyArgs {

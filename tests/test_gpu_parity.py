@@ -382,3 +382,27 @@ def test_gpu_packer_matches_host_pipeline(prune):
         layer_cpu.pack(torch.from_numpy(w).half())
         assert torch.equal(layer_gpu.meta.cpu(), layer_cpu.meta)
         assert torch.equal(layer_gpu.packed_binary_sparse.cpu(), layer_cpu.packed_binary_sparse)
+
+
+def test_unaligned_c_and_d_use_the_direct_epilogue():
+    """C and D that are only 2-byte / 4-byte aligned (the 16-byte epilogue cannot be used)."""
+    m, n, k = 512, 128, 256
+    a, meta = synthetic.make_weight(m, k, seed=51)
+    bi = synthetic.make_b(k, n, seed=52, kind="int")
+    c = torch.randint(-8, 9, (m, n)).to(torch.float16)
+    dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
+    ad, md, bd = _gpu(a, meta, bi)
+    prep = _native.prepare(ad, md, m, k)
+    for dtype in (torch.float16, torch.float32):
+        exact = oracle.host_gemm(dense, bi.numpy(), c=c.numpy(), alpha=1.0, beta=1.0,
+                                 d_dtype=oracle.F16 if dtype == torch.float16 else oracle.F32)
+        d_store = torch.zeros(m * n + 8, dtype=dtype, device="cuda")
+        d = d_store[1:1 + m * n].view(m, n)
+        c_store = torch.zeros(m * n + 8, dtype=torch.float16, device="cuda")
+        cd = c_store[1:1 + m * n].view(m, n)
+        cd.copy_(c.cuda())
+        assert d.data_ptr() % 16 != 0 and cd.data_ptr() % 16 != 0
+        _native.matmul_prepared(prep, bd, d, m, n, k, c=cd, alpha=1.0, beta=1.0)
+        torch.cuda.synchronize()
+        assert np.array_equal(d.cpu().numpy(), exact)
+        assert float(d_store[0]) == 0.0 and float(d_store[1 + m * n]) == 0.0  # nothing written outside D
