@@ -249,6 +249,10 @@ __device__ __forceinline__ void compute_stage(const char* stage_lds, const AChun
 #ifndef ONEBIT_MAIN_INTERLEAVE /* 1: force the order SMFMAC, LDS read, VALU inside each K-step region */
 #define ONEBIT_MAIN_INTERLEAVE 0
 #endif
+#ifndef ONEBIT_EXP_EXTRA  /* marginal-cost probes, data unchanged: 1: every sign expansion is computed twice,
+                             2: every transpose read is issued twice, 3: every B copy is issued twice */
+#define ONEBIT_EXP_EXTRA 0
+#endif
 #ifndef ONEBIT_EXP_NO_BARRIER
 #define ONEBIT_EXP_NO_BARRIER 0
 #endif
@@ -275,6 +279,12 @@ __device__ __forceinline__ void load_b_frags(const char* stage_lds, int ks, half
       const u32x2_t t = lds_read_tr16(stage_lds + lane_row_off + row_const * (BN * 2) + frag_off[fn]);
       raw[2 * q] = t.x;
       raw[2 * q + 1] = t.y;
+      if (ONEBIT_EXP_EXTRA == 2) {
+        int again = lane_row_off;
+        asm volatile("" : "+v"(again));
+        const u32x2_t t2 = lds_read_tr16(stage_lds + again + row_const * (BN * 2) + frag_off[fn]);
+        asm volatile("" ::"v"(t2));
+      }
     }
     bv[fn] = __builtin_bit_cast(half16_t, raw);
   }
@@ -288,7 +298,15 @@ __device__ __forceinline__ void expand_frags(const AChunk (&a)[FM], uint32_t one
     return;
   }
 #pragma unroll
-  for (int fm = 0; fm < FM; ++fm) av[fm] = expand_signs<STEP>(a[fm], one);
+  for (int fm = 0; fm < FM; ++fm) {
+    av[fm] = expand_signs<STEP>(a[fm], one);
+    if (ONEBIT_EXP_EXTRA == 1) {
+      AChunk again = a[fm];
+      asm volatile("" : "+v"(again.sign));
+      const half8_t av2 = expand_signs<STEP>(again, one);
+      asm volatile("" ::"v"(av2));
+    }
+  }
 }
 
 template <int STEP, int FM, int FN>
@@ -407,8 +425,10 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
       if (next_k0 + kStageK <= p.k) {  // wave-uniform: a full stage
 #pragma unroll
         for (int i = 0; i < NL; ++i)
-          if (ONEBIT_EXP_COPY_MODE != 5 || (i & 1) == 0)
+          if (ONEBIT_EXP_COPY_MODE != 5 || (i & 1) == 0) {
             lds_dma16_base(b_stage, b_off[i], lds_dst[i] + ring * TS::STAGE_BYTES);
+            if (ONEBIT_EXP_EXTRA == 3) lds_dma16_base(b_stage, b_off[i], lds_dst[i] + ring * TS::STAGE_BYTES);
+          }
       } else {
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
