@@ -90,7 +90,7 @@ const char *onebit_sparse_last_error(void);
  * shapes with n <= 16 use the split-K kernel (1, default) or the main kernel (0). Process-wide. */
 void onebit_sparse_set_tile_config(int tile_config);
 void onebit_sparse_set_skinny_enabled(int enabled);
-/* Weight rows one workgroup of the split-K kernel covers: 32 or 64; <= 0 = automatic. */
+/* Weight rows one workgroup of the split-K kernel covers: 32, 64 or 128; <= 0 = automatic. */
 void onebit_sparse_set_skinny_rows(int rows);
 
 /* Diagnostic, no counterpart in the reference: sustained rate of v_smfmac_f32_32x32x32_f16 in a register-only

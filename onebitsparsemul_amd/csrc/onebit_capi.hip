@@ -107,7 +107,9 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
     args.c_f16 = c_dtype == ONEBIT_DTYPE_F16;
     args.d_f16 = d_dtype == ONEBIT_DTYPE_F16;
     int rows = g_skinny_rows.load();
-    if (rows <= 0) rows = (m / 64 >= 128) ? 64 : 32;  // 64-row groups once they give at least 128 workgroups
+    // the largest row group that still gives about two workgroups per three compute units (measured: larger groups
+    // re-read B less often, but idle compute units cost more)
+    if (rows <= 0) rows = (m / 128 >= 160) ? 128 : (m / 64 >= 160) ? 64 : 32;
     ONEBIT_HIP(onebit::launch_skinny(args, rows, stream));
     return ONEBIT_OK;
   }

@@ -681,138 +681,195 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
 
 // =====================================================================================================
 // skinny_kernel: N <= 16 (decode shapes). HBM-bound: every byte of the prepared operand is read once.
-// Workgroup = 16 wavefronts that share R row blocks (32 rows each) and split K among themselves: wavefront w
-// takes the K chunks (of 256) w, w+16, w+32, ... Each wavefront stages the B rows of its chunk in a private
-// 8 KiB LDS region as a zero-padded [256][16] fp16 image, feeds them to SMFMAC through transpose reads and
-// keeps a 32x32 fp32 partial tile per row block. The sixteen partial tiles are added through LDS in
-// wavefront order (deterministic) and the epilogue is applied. grid = M / (32 R) workgroups; no global
-// workspace, no atomics.
+// Workgroup = NW wavefronts that share R row blocks (32 rows each) and split K among themselves: wavefront w
+// takes the K chunks (of 256) w, w + NW, w + 2 NW, ... Each wavefront stages the B rows of its chunk in a private
+// 8 KiB LDS region as a zero-padded [256][16] fp16 image, feeds them to SMFMAC through transpose reads (one
+// fragment serves the R row blocks) and keeps a 32x32 fp32 partial tile per row block. The prepared operand and
+// the B rows of the wavefront's next chunk are loaded into registers while the current chunk is multiplied.
+// Wavefronts never wait for one another inside the K loop (LDS operations of one wavefront execute in order).
+// The NW partial tiles of a row block are added through LDS in wavefront order (deterministic) and the epilogue
+// is applied. grid = M / (32 R) workgroups; no global workspace, no atomics.
 // =====================================================================================================
-constexpr int kSkinnyWaves = 16;
-constexpr int kSkinnyRegion = kChunkK * 16 * 2;  // bytes of one wavefront's B image
+#ifndef ONEBIT_EXP_SKINNY
+#define ONEBIT_EXP_SKINNY 0  // measurement builds (results wrong): 1 no B reloads, 2 one fragment group per chunk, 3 one expansion per chunk, 4 loads and image stores only
+#endif
+constexpr int kSkinnyRegion = kChunkK * 16 * 2;  // bytes of one B image
+constexpr int kSkinnyTileBytes = kRowBlock * 16 * 4;
 
-template <int R>
-__global__ __launch_bounds__(1024) void skinny_kernel(SkinnyArgs p) {
-  static_assert(R * 32 * 16 * 4 <= kSkinnyRegion, "partial tiles must fit the wavefront's LDS region");
-  __shared__ __attribute__((aligned(16))) char bs[kSkinnyWaves * kSkinnyRegion];
+enum SkinnyBMode { kSkinnyB16 = 0, kSkinnyB8 = 1, kSkinnyB4 = 2, kSkinnyBScalar = 3 };
+
+// 16-byte piece q of the image of the chunk at k_base: row q / 2, columns 8 (q % 2) ... + 7; zero outside B.
+// Vector modes only (n = 16, 8 or 4 with B aligned to its row size).
+__device__ __forceinline__ u32x4_t skinny_load_piece(const _Float16* __restrict__ b, int n, int mode, int k_base,
+                                                      int rows_valid, int q) {
+  const int row = q >> 1, h = q & 1;
+  const bool ok = row < rows_valid;
+  const char* base = reinterpret_cast<const char*>(b);
+  u32x4_t v = u32x4_t{0, 0, 0, 0};
+  if (mode == kSkinnyB16) {
+    const char* src = ok ? base + ((size_t)k_base * 16 + (size_t)q * 8) * 2 : base;
+    v = *reinterpret_cast<const u32x4_t*>(src);
+    if (!ok) v = u32x4_t{0, 0, 0, 0};
+  } else if (mode == kSkinnyB8) {
+    const bool use = ok && h == 0;
+    const char* src = use ? base + (size_t)(k_base + row) * 16 : base;
+    v = *reinterpret_cast<const u32x4_t*>(src);
+    if (!use) v = u32x4_t{0, 0, 0, 0};
+  } else {  // kSkinnyB4
+    const bool use = ok && h == 0;
+    const char* src = use ? base + (size_t)(k_base + row) * 8 : base;
+    const u32x2_t t = *reinterpret_cast<const u32x2_t*>(src);
+    if (use) v = u32x4_t{t.x, t.y, 0, 0};
+  }
+  return v;
+}
+
+template <int NW, int R, int MODE>
+__global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(SkinnyArgs p) {
+  constexpr int NT = 64 * NW;
+  static_assert(R * kSkinnyTileBytes <= kSkinnyRegion, "partial tiles reuse the wavefront's image memory");
+  __shared__ __attribute__((aligned(16))) char bs[NW * kSkinnyRegion];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int rb_total = p.m / kRowBlock;
   const int rb_first = blockIdx.x * R;
   char* region = bs + wave * kSkinnyRegion;
+  // kernel arguments the lambdas use, as values (capturing the argument struct would move it to scratch memory)
+  const _Float16* __restrict__ b_ptr = p.b;
+  const uint8_t* __restrict__ prep = p.prep;
+  const int n_cols = p.n, k_rows = p.k, kc_total = p.kc_total;
+
+  auto load_a = [&](int kc, AChunk (&a)[R]) __attribute__((always_inline)) {
+    if (kc >= kc_total) kc = kc_total - 1;  // never multiplied
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      int rb = rb_first + r;
+      if (rb >= rb_total) rb = rb_total - 1;  // never stored
+      a[r] = load_a_chunk(prep + ((size_t)rb * kc_total + kc) * kBlockBytes, lane);
+    }
+  };
+  auto rows_valid_of = [&](int k_base) __attribute__((always_inline)) {
+    const int rows = k_rows - k_base;
+    return rows < 0 ? 0 : (rows > kChunkK ? kChunkK : rows);
+  };
+  // vector modes: the image of a chunk travels through registers, loaded while the previous chunk is multiplied;
+  // element mode (any n, any alignment): loaded and stored in one go when the image is due, piece by piece
+  auto load_b = [&](int kc, u32x4_t (&v)[8]) __attribute__((always_inline)) {
+    if (MODE == kSkinnyBScalar) return;
+    const int k_base = kc * kChunkK;
+    const int rows_valid = rows_valid_of(k_base);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = skinny_load_piece(b_ptr, n_cols, MODE, k_base, rows_valid, lane + i * 64);
+  };
+  auto store_b = [&](int kc, const u32x4_t (&v)[8]) __attribute__((always_inline)) {
+    if (MODE == kSkinnyBScalar) {
+      // the chunk's rows are one run of 256 n elements; rows at or past K are written as zeros, the padding
+      // columns n ... 15 keep the zeros the image was cleared to
+      const int k_base = kc * kChunkK;
+      const int valid = rows_valid_of(k_base) * n_cols, total = kChunkK * n_cols;
+      const _Float16* src = b_ptr + (size_t)k_base * n_cols;
+      for (int e0 = lane; e0 < total; e0 += 64 * 4) {
+        uint16_t bits[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int e = e0 + i * 64;
+          bits[i] = __builtin_bit_cast(uint16_t, e < valid ? src[e] : b_ptr[0]);
+          if (e >= valid) bits[i] = 0;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int e = e0 + i * 64;
+          if (e < total) *reinterpret_cast<uint16_t*>(region + (e / n_cols) * 32 + (e % n_cols) * 2) = bits[i];
+        }
+      }
+      return;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4_t*>(region + (lane + i * 64) * 16) = v[i];
+  };
 
   float16_t acc[R];
 #pragma unroll
   for (int r = 0; r < R; ++r)
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[r][v] = 0.f;
-
   const uint32_t one = packed_one_in_vgpr();
   const int i16 = lane & 15, gb = lane >> 5;
   // lanes 16-31 and 48-63 would hold columns 16-31: they re-read columns 0-15 and are never stored
   const char* lane_ptr = region + (8 * gb + (i16 >> 2)) * 32 + (i16 & 3) * 8;
-  const bool vector_b = p.n == 16 && (reinterpret_cast<uintptr_t>(p.b) & 15) == 0;
-  const bool vector8_b = (p.n == 4 || p.n == 8) && (reinterpret_cast<uintptr_t>(p.b) & 15) == 0;
 
-  for (int kc = wave; kc < p.kc_total; kc += kSkinnyWaves) {
-    AChunk a[R];
+  auto frag = [&](int st) __attribute__((always_inline)) {
+    u32x8_t raw;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      int rb = rb_first + r;
-      if (rb >= rb_total) rb = rb_total - 1;
-      a[r] = load_a_chunk(p.prep + ((size_t)rb * p.kc_total + kc) * kBlockBytes, lane);
+    for (int q = 0; q < 4; ++q) {
+      const int row_const = st * 32 + 4 * (q & 1) + 16 * (q >> 1);
+      const u32x2_t t = lds_read_tr16(lane_ptr + row_const * 32);
+      raw[2 * q] = t.x;
+      raw[2 * q + 1] = t.y;
     }
-    const int k_base = kc * kChunkK;
-    const int rows_valid = (p.k - k_base) < kChunkK ? (p.k - k_base) : kChunkK;  // >= 1
-    if (vector_b) {
-      // the chunk's rows are 8 KiB of consecutive memory: eight 16-byte pieces per lane
-      const u32x4_t* src = reinterpret_cast<const u32x4_t*>(p.b + (size_t)k_base * 16);
-      u32x4_t v[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int idx = lane + i * 64;
-        const bool ok = (idx >> 1) < rows_valid;
-        v[i] = src[ok ? idx : 0];
-        if (!ok) v[i] = u32x4_t{0, 0, 0, 0};
-      }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4_t*>(region + (lane + i * 64) * 16) = v[i];
-    } else if (vector8_b) {
-      // n == 4 (or n == 8): a row is 8 (16) bytes; four rows per lane, padded to the 32-byte LDS rows
-#pragma unroll
-      for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4_t*>(region + (lane + i * 64) * 16) = u32x4_t{0, 0, 0, 0};
-      const int row_bytes = p.n * 2;
-      const char* src = reinterpret_cast<const char*>(p.b) + (size_t)k_base * row_bytes;
-      u32x4_t v[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int row = lane + i * 64;
-        const char* q = src + (size_t)(row < rows_valid ? row : 0) * row_bytes;
-        if (p.n == 4) {
-          const u32x2_t t = *reinterpret_cast<const u32x2_t*>(q);
-          v[i] = u32x4_t{t.x, t.y, 0, 0};
-        } else {
-          v[i] = *reinterpret_cast<const u32x4_t*>(q);
-        }
-        if (row >= rows_valid) v[i] = u32x4_t{0, 0, 0, 0};
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4_t*>(region + (lane + i * 64) * 32) = v[i];
-    } else {
-      // any n <= 16, any alignment: the valid part of the chunk is one run of rows_valid * n elements
-#pragma unroll
-      for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4_t*>(region + (lane + i * 64) * 16) = u32x4_t{0, 0, 0, 0};
-      const _Float16* src = p.b + (size_t)k_base * p.n;
-      const int total = rows_valid * p.n;
-      constexpr int BATCH = 8;
-      for (int e0 = lane; e0 < total; e0 += 64 * BATCH) {
-        _Float16 v[BATCH];
-#pragma unroll
-        for (int i = 0; i < BATCH; ++i) {
-          const int e = e0 + i * 64;
-          v[i] = src[e < total ? e : 0];
-        }
-#pragma unroll
-        for (int i = 0; i < BATCH; ++i) {
-          const int e = e0 + i * 64;
-          if (e < total) *reinterpret_cast<_Float16*>(region + (e / p.n) * 32 + (e % p.n) * 2) = v[i];
-        }
-      }
-    }
-    // the region is private to this wavefront and its LDS operations execute in order: no barrier needed
-
-    // all B fragments of the chunk first (32 transpose reads in flight), then the SMFMACs back to back
-    half16_t bfrag[kStepsPerChunk];
-#pragma unroll
-    for (int st = 0; st < kStepsPerChunk; ++st) {
-      u32x8_t raw;
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int row_const = st * 32 + 4 * (q & 1) + 16 * (q >> 1);
-        const u32x2_t t = lds_read_tr16(lane_ptr + row_const * 32);
-        raw[2 * q] = t.x;
-        raw[2 * q + 1] = t.y;
-      }
-      bfrag[st] = __builtin_bit_cast(half16_t, raw);
-    }
-    auto step = [&](auto step_tag) {
+    return __builtin_bit_cast(half16_t, raw);
+  };
+  auto compute = [&](const AChunk (&a)[R]) __attribute__((always_inline)) {
+    // FG fragments (4 FG transpose reads) in flight, then their SMFMACs back to back; the scheduling barriers keep
+    // the next group's reads from being hoisted (8 registers per fragment)
+    constexpr int FG = R >= 4 ? 2 : 4;
+    half16_t bfrag[FG];
+    auto step = [&](auto step_tag) __attribute__((always_inline)) {
       constexpr int STEP = decltype(step_tag)::value;
 #pragma unroll
       for (int r = 0; r < R; ++r)
-        acc[r] = smfmac_step<STEP, false>(a[r], expand_signs<STEP>(a[r], one), bfrag[STEP], acc[r]);
+#if ONEBIT_EXP_SKINNY == 3
+        acc[r] = smfmac_step<STEP, false>(a[r], expand_signs<0>(a[0], one), bfrag[STEP % FG], acc[r]);
+#else
+        acc[r] = smfmac_step<STEP, false>(a[r], expand_signs<STEP>(a[r], one), bfrag[STEP % FG], acc[r]);
+#endif
     };
-    step(std::integral_constant<int, 0>{});
-    step(std::integral_constant<int, 1>{});
-    step(std::integral_constant<int, 2>{});
-    step(std::integral_constant<int, 3>{});
-    step(std::integral_constant<int, 4>{});
-    step(std::integral_constant<int, 5>{});
-    step(std::integral_constant<int, 6>{});
-    step(std::integral_constant<int, 7>{});
+    auto group = [&](auto first_tag) __attribute__((always_inline)) {
+      constexpr int FIRST = decltype(first_tag)::value;
+#if ONEBIT_EXP_SKINNY == 2
+      if (FIRST == 0)
+#endif
+#pragma unroll
+      for (int st = 0; st < FG; ++st) bfrag[st] = frag(FIRST + st);
+      step(std::integral_constant<int, FIRST>{});
+      step(std::integral_constant<int, FIRST + 1>{});
+      if constexpr (FG == 4) {
+        step(std::integral_constant<int, FIRST + 2>{});
+        step(std::integral_constant<int, FIRST + 3>{});
+      }
+      if (FIRST + FG < kStepsPerChunk) __builtin_amdgcn_sched_barrier(0);
+    };
+    group(std::integral_constant<int, 0>{});
+    if constexpr (FG == 2) group(std::integral_constant<int, 2>{});
+    group(std::integral_constant<int, 4>{});
+    if constexpr (FG == 2) group(std::integral_constant<int, 6>{});
+  };
+
+  // sixteen wavefronts leave 128 registers each: no room to hold the next image (32 registers) during the SMFMACs
+  constexpr bool kPrefetchB = NW <= 8 && MODE != kSkinnyBScalar;
+  u32x4_t breg[8];
+  AChunk a_cur[R], a_next[R];
+  if (kPrefetchB) load_b(wave, breg);
+  load_a(wave, a_cur);
+  for (int kc = wave; kc < kc_total; kc += NW) {
+    if (!kPrefetchB) load_b(kc, breg);
+    store_b(kc, breg);  // after the previous chunk's fragment reads: LDS operations of a wavefront execute in order
+#if ONEBIT_EXP_SKINNY != 1
+    if (kPrefetchB) load_b(kc + NW, breg);
+#endif
+    load_a(kc + NW, a_next);
+#if ONEBIT_EXP_SKINNY == 4
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r][0] += __builtin_bit_cast(float, a_cur[r].meta.x ^ a_cur[r].sign.y);
+#else
+    compute(a_cur);
+#endif
+#pragma unroll
+    for (int r = 0; r < R; ++r) a_cur[r] = a_next[r];
   }
 
   smfmac_drain();
-  // ---- add the sixteen partial tiles through LDS: region of wavefront w := its R tiles as [r][32 rows][16 cols] fp32
+  // ---- add the NW partial tiles through LDS: region of wavefront w := its R tiles as [r][32 rows][16 cols] fp32
   {
     float* tile = reinterpret_cast<float*>(region);
     const int col = lane & 31;
@@ -827,10 +884,10 @@ __global__ __launch_bounds__(1024) void skinny_kernel(SkinnyArgs p) {
     }
   }
   __syncthreads();
-  for (int idx = tid; idx < R * 32 * 16; idx += 1024) {
+  for (int idx = tid; idx < R * kRowBlock * 16; idx += NT) {
     float sum = 0.f;
 #pragma unroll
-    for (int w = 0; w < kSkinnyWaves; ++w) sum += reinterpret_cast<const float*>(bs + w * kSkinnyRegion)[idx];
+    for (int w = 0; w < NW; ++w) sum += reinterpret_cast<const float*>(bs + w * kSkinnyRegion)[idx];
     const int col = idx & 15;
     const int row = rb_first * kRowBlock + (idx >> 4);
     if (col < p.n && row < p.m) {
@@ -908,17 +965,27 @@ hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
   }
 }
 
-template <int R>
-static hipError_t launch_skinny_cfg(const SkinnyArgs& args, hipStream_t stream) {
+template <int NW, int R, int MODE>
+static hipError_t launch_skinny_mode(const SkinnyArgs& args, hipStream_t stream) {
   const int row_blocks = args.m / kRowBlock;
-  hipLaunchKernelGGL((skinny_kernel<R>), dim3((row_blocks + R - 1) / R), dim3(1024), 0, stream, args);
+  hipLaunchKernelGGL((skinny_kernel<NW, R, MODE>), dim3((row_blocks + R - 1) / R), dim3(64 * NW), 0, stream, args);
   return hipGetLastError();
+}
+
+template <int NW, int R>
+static hipError_t launch_skinny_cfg(const SkinnyArgs& args, hipStream_t stream) {
+  const uintptr_t address = reinterpret_cast<uintptr_t>(args.b);
+  if (args.n == 16 && (address & 15) == 0) return launch_skinny_mode<NW, R, kSkinnyB16>(args, stream);
+  if (args.n == 8 && (address & 15) == 0) return launch_skinny_mode<NW, R, kSkinnyB8>(args, stream);
+  if (args.n == 4 && (address & 7) == 0) return launch_skinny_mode<NW, R, kSkinnyB4>(args, stream);
+  return launch_skinny_mode<NW, R, kSkinnyBScalar>(args, stream);
 }
 
 hipError_t launch_skinny(SkinnyArgs args, int rows_per_group, hipStream_t stream) {
   switch (rows_per_group) {
-    case 32: return launch_skinny_cfg<1>(args, stream);
-    case 64: return launch_skinny_cfg<2>(args, stream);
+    case 32: return launch_skinny_cfg<16, 1>(args, stream);  // sixteen wavefronts split K: small M
+    case 64: return launch_skinny_cfg<8, 2>(args, stream);
+    case 128: return launch_skinny_cfg<8, 4>(args, stream);
     default: return hipErrorInvalidValue;
   }
 }

@@ -36,7 +36,7 @@ hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream);
 // dense fp16 (m x k) -> one-bit values `a` and metadata `e`; prune != 0 applies the 2:4 magnitude mask first
 hipError_t launch_pack(const void* w, void* a, void* e, int m, int k, int prune, int layout, hipStream_t stream);
 
-// Split-K kernel for n <= 16; rows_per_group (32 or 64) = weight rows one workgroup covers.
+// Split-K kernel for n <= 16; rows_per_group (32, 64 or 128) = weight rows one workgroup covers.
 constexpr int kSkinnyMaxN = 16;
 hipError_t launch_skinny(SkinnyArgs args, int rows_per_group, hipStream_t stream);
 

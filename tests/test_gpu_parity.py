@@ -24,9 +24,11 @@ REL_TOL = 1e-3  # stated by the task for fp16 B: rel-err <= 1e-3
 def _defaults():
     _native.set_tile_config(-1)
     _native.set_skinny_enabled(True)
+    _native.set_skinny_rows(-1)
     yield
     _native.set_tile_config(-1)
     _native.set_skinny_enabled(True)
+    _native.set_skinny_rows(-1)
 
 
 def _gpu(*ts):
@@ -185,6 +187,24 @@ def test_config3_decode(m, k, n):
         assert np.array_equal(_run_prepared(a, meta, bi, m, n, k, out_dtype=torch.float32), exact)
         assert np.array_equal(_run_prepared(a, meta, bi, m, n, k, out_dtype=torch.float16), exact.astype(np.float16))
         _assert_close(_run_prepared(a, meta, b, m, n, k), ref64)
+
+
+@pytest.mark.parametrize("rows", [32, 64, 128])
+@pytest.mark.parametrize("m,n,k", [(64, 1, 32), (192, 5, 800), (320, 8, 4128), (4096, 16, 4096), (1088, 4, 2048),
+                                   (2240, 16, 8224), (128, 13, 12320)])
+def test_split_k_workgroup_shapes(rows, m, n, k):
+    """every row-group size of the split-K kernel: chunk counts that do not divide among the wavefronts, a row
+    group past the last row block, K tails, every B staging mode (n = 16, 8, 4 vector copies; element copies)"""
+    _native.set_skinny_rows(rows)
+    a, meta = synthetic.make_weight(m, k, seed=rows + m + k)
+    dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
+    bi = synthetic.make_b(k, n, seed=n, kind="int")
+    ci = synthetic.make_c(m, n, seed=n + 1, dtype=torch.float32).round()
+    exact = oracle.host_gemm(dense, bi.numpy(), c=ci.numpy(), alpha=2.0, beta=1.0, d_dtype=oracle.F32, acc="f32")
+    got = _run_prepared(a, meta, bi, m, n, k, c=ci, alpha=2.0, beta=1.0, out_dtype=torch.float32)
+    assert np.array_equal(got, exact)
+    b = synthetic.make_b(k, n, seed=n + 50, kind="normal")
+    _assert_close(_run_prepared(a, meta, b, m, n, k), oracle.blas_matmul(dense, b.numpy()))
 
 
 def test_config3_split_k_is_deterministic_and_reusable():
