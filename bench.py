@@ -24,9 +24,9 @@ DENSE_F16_PEAK_TFLOPS = CU_COUNT * CLOCK_HZ * 4096 / 1e12        # 2516.6: publi
 SMFMAC_PEAK_TFLOPS = 2 * DENSE_F16_PEAK_TFLOPS                   # dense-equivalent rate of v_smfmac f16
 HBM_PEAK_GBS = 8000.0
 # HBM-side bytes per launch of the dominant kernel, from two rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE), each
-# scaled by what the same counter reads for a 256 MiB copy kernel (x2.000 and x1.000): see
+# scaled by what the same counter reads for an elementwise copy kernel over 256 MiB (x2.000 and x1.000): see
 # profiles/gemm_kernel_square8192_counters.txt. Only the workload it was measured on has a figure.
-MEASURED_TRAFFIC_BYTES = {"square:8192": (319276 * 2.000 + 180082 * 1.000) * 1024}
+MEASURED_TRAFFIC_BYTES = {"square:8192": (262314.7 * 2.000 + 131072.0 * 1.000) * 1024}
 
 
 def parse_workload(text):
@@ -163,7 +163,7 @@ def main():
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-ceiling", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
-                    help="also run one 256 MiB device-to-device copy kernel (reference point for HBM counters)")
+                    help="also run one elementwise copy kernel over 256 MiB (reference point for HBM counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
@@ -185,9 +185,10 @@ def main():
         return
 
     if args.calibration_copy:
-        src = torch.zeros(128 << 20, dtype=torch.float16, device="cuda")
+        # a plain elementwise kernel of known size: reads 256 MiB, writes 256 MiB (grid 128 Mi elements / 1024 per block)
+        src = torch.randn(128 << 20, dtype=torch.float16, device="cuda")
         dst = torch.empty_like(src)
-        dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        torch.neg(src, out=dst)
         torch.cuda.synchronize()
         del src, dst
     kernel_s, wall_s, operands = run_gemm(w, args.steps, args.warmup)
