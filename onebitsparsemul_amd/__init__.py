@@ -113,8 +113,8 @@ class PreparedWeight:
 
 
 class BinaryLinear_2_4(nn.Module):
-    """1-bit 2:4 sparse linear layer without bias: y = x @ W.T, W (outfeatures, infeatures) stored at 1.5 bits
-    per weight. Reference: onebit_sparse_mul/__init__.py:101-145."""
+    """1-bit 2:4 sparse linear layer: y = x @ W.T (+ bias when one has been assigned), W (outfeatures, infeatures)
+    stored at 1.5 bits per weight. Reference: onebit_sparse_mul/__init__.py:101-145."""
 
     def __init__(self, infeatures: int, outfeatures: int):
         super().__init__()
@@ -126,6 +126,7 @@ class BinaryLinear_2_4(nn.Module):
         self.register_buffer("meta", torch.zeros((outfeatures, infeatures // 16), dtype=torch.int16))
         self.vaild = False
         self._prepared = None
+        self.bias = None  # optional (outfeatures,) tensor added to the output; the model script assigns it
 
     def pack(self, weight):
         """weight (outfeatures, infeatures): prune to 2:4 by magnitude, keep the signs.
@@ -161,4 +162,7 @@ class BinaryLinear_2_4(nn.Module):
         lead = x.shape[:-1]
         b = x.reshape(-1, self.infeatures).to(torch.float16).T.contiguous()  # (k, batch)
         out = self._prepared.matmul(b, out_dtype=torch.float16)           # (outfeatures, batch)
-        return out.T.reshape(*lead, self.outfeatures).to(x.dtype)
+        y = out.T.reshape(*lead, self.outfeatures).to(x.dtype)
+        if self.bias is not None:
+            y = y + self.bias.to(y.dtype)
+        return y
