@@ -92,6 +92,11 @@ void onebit_sparse_set_tile_config(int tile_config);
 void onebit_sparse_set_skinny_enabled(int enabled);
 /* Weight rows one workgroup of the split-K kernel covers: 32, 64 or 128; <= 0 = automatic. */
 void onebit_sparse_set_skinny_rows(int rows);
+/* K splits of the main kernel (n > 16): 1 = never split, N > 1 = N splits (at most one per 256 of K), <= 0 =
+ * automatic (few tiles and a long K). A split call writes fp32 partial sums to a library-owned buffer kept per
+ * device and stream (grown with hipMalloc on first use: warm up before capturing the call in a HIP graph) and adds
+ * them in split order, so results do not depend on timing. */
+void onebit_sparse_set_split_k(int splits);
 
 /* Diagnostic, no counterpart in the reference: sustained rate of v_smfmac_f32_32x32x32_f16 in a register-only
  * loop on the current device (one wavefront per SIMD, `iterations` x 16 instructions each), in dense-equivalent

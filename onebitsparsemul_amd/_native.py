@@ -15,7 +15,8 @@ META_REFERENCE, META_CUTLASS, META_LOGICAL = 0, 1, 2
 EXPORTS = (
     "onebit_sparse_matmul", "onebit_sparse_matmul_ex", "onebit_sparse_prepared_bytes", "onebit_sparse_prepare",
     "onebit_sparse_matmul_prepared", "onebit_sparse_pack", "onebit_sparse_last_error", "onebit_sparse_set_tile_config",
-    "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_measure_smfmac_rate",
+    "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_set_split_k",
+    "onebit_sparse_measure_smfmac_rate",
 )
 
 _lib = None
@@ -48,6 +49,8 @@ def lib():
         L.onebit_sparse_set_skinny_enabled.argtypes = [i32]
         L.onebit_sparse_set_skinny_rows.restype = None
         L.onebit_sparse_set_skinny_rows.argtypes = [i32]
+        L.onebit_sparse_set_split_k.restype = None
+        L.onebit_sparse_set_split_k.argtypes = [i32]
         L.onebit_sparse_measure_smfmac_rate.restype = i32
         L.onebit_sparse_measure_smfmac_rate.argtypes = [i32, i32, ctypes.POINTER(ctypes.c_double)]
         _lib = L
@@ -149,6 +152,10 @@ def set_skinny_enabled(flag):
 
 def set_skinny_rows(rows):
     lib().onebit_sparse_set_skinny_rows(rows)
+
+
+def set_split_k(splits):
+    lib().onebit_sparse_set_split_k(splits)
 
 
 def measure_smfmac_rate(random_operands=True, iterations=50000):

@@ -9,6 +9,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
+#include <map>
 #include <mutex>
 #include <string>
 
@@ -18,6 +19,7 @@ thread_local std::string g_last_error;
 std::atomic<int> g_tile_config{-1};
 std::atomic<int> g_skinny_enabled{1};
 std::atomic<int> g_skinny_rows{-1};
+std::atomic<int> g_split_k{-1};
 
 int fail(int code, const char* fmt, ...) {
   char buf[512];
@@ -40,10 +42,17 @@ constexpr int kMaxDevices = 64;
 
 // Library-owned device memory: the reordered operand of the one-call entry points. Grow-only, one per
 // device, freed at process exit by the runtime. Work that uses it is ordered by the caller's stream.
+struct Buffer {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+};
 struct DeviceState {
   std::mutex mu;
   void* prep = nullptr;
   size_t prep_bytes = 0;
+  // fp32 partial sums of the K-split passes: one buffer per stream, so that calls on different streams do not
+  // share one (calls on the same stream are ordered)
+  std::map<hipStream_t, Buffer> split_ws;
 };
 DeviceState g_dev[kMaxDevices];
 
@@ -89,6 +98,34 @@ int pick_tile(int m, int n) {
   return onebit::kTile128x128s;
 }
 
+// Number of K splits for the main kernel. Few tiles and a long K leave most compute units idle and make the
+// time the length of one workgroup's K loop; splitting K fills the GPU at the price of a second launch and of
+// writing and re-reading fp32 partial sums. Chosen with a cost model fitted to measurements of the 128 x 128
+// tile on MI355X (microseconds): 1.4 per 256-wide chunk of one workgroup's K loop, times the rounds of 512
+// resident workgroups; a split adds 5 for the second launch and the partial sums move at about 1.5 TB/s.
+int pick_splits(int m, int n, int k, int tile) {
+  const int chunks = (k + onebit::kChunkK - 1) / onebit::kChunkK;
+  const int forced = g_split_k.load();
+  if (forced >= 1) return forced < chunks ? forced : chunks;
+  if (tile != onebit::kTile128x128s) return 1;
+  const double tiles = (double)((m + 127) / 128) * ((n + 127) / 128);
+  const double result_bytes = 4.0 * m * n;
+  int best = 1;
+  double best_us = 1e30;
+  for (int s : {1, 2, 3, 4, 6, 8, 12, 16}) {
+    if (s > chunks) break;
+    const int per_split = (chunks + s - 1) / s;
+    const double rounds = (double)(long)((tiles * s + 511) / 512);
+    double us = 1.4 * per_split * rounds;
+    if (s > 1) us += 5.0 + (s + 1) * result_bytes / 1.5e6;
+    if (us < best_us) {
+      best_us = us;
+      best = s;
+    }
+  }
+  return best;
+}
+
 int matmul_prepared_impl(const void* prepared, const void* b, const void* c, void* d, int m, int n, int k, float alpha,
                          float beta, int c_dtype, int d_dtype, hipStream_t stream) {
   if (!prepared || !b || !d) return fail(ONEBIT_ERR_ARGUMENT, "null operand pointer");
@@ -124,7 +161,24 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
   args.alpha = alpha; args.beta = beta;
   args.c_f16 = c_dtype == ONEBIT_DTYPE_F16;
   args.d_f16 = d_dtype == ONEBIT_DTYPE_F16;
-  ONEBIT_HIP(onebit::launch_gemm(args, pick_tile(m, n), stream));
+  const int tile = pick_tile(m, n);
+  const int splits = pick_splits(m, n, k, tile);
+  if (splits > 1) {
+    const int cps = (kc_total + splits - 1) / splits;
+    args.chunks_per_split = cps;
+    args.splits = (kc_total + cps - 1) / cps;  // every split non-empty
+    int device = 0;
+    ONEBIT_HIP(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) return fail(ONEBIT_ERR_ARGUMENT, "device ordinal %d not supported", device);
+    DeviceState& st = g_dev[device];
+    std::lock_guard<std::mutex> lock(st.mu);
+    Buffer& ws = st.split_ws[stream];
+    if (int rc = grow(&ws.ptr, &ws.bytes, (size_t)args.splits * m * n * sizeof(float)); rc != ONEBIT_OK) return rc;
+    args.split_ws = static_cast<float*>(ws.ptr);
+    ONEBIT_HIP(onebit::launch_gemm(args, tile, stream));
+    return ONEBIT_OK;
+  }
+  ONEBIT_HIP(onebit::launch_gemm(args, tile, stream));
   return ONEBIT_OK;
 }
 
@@ -137,6 +191,7 @@ const char* onebit_sparse_last_error(void) { return g_last_error.c_str(); }
 void onebit_sparse_set_tile_config(int tile_config) { g_tile_config.store(tile_config); }
 void onebit_sparse_set_skinny_enabled(int enabled) { g_skinny_enabled.store(enabled ? 1 : 0); }
 void onebit_sparse_set_skinny_rows(int rows) { g_skinny_rows.store(rows); }
+void onebit_sparse_set_split_k(int splits) { g_split_k.store(splits); }
 
 size_t onebit_sparse_prepared_bytes(int m, int k) {
   if (m <= 0 || k <= 0) return 0;

@@ -393,6 +393,10 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
 
   const int stages_total = (p.k + kStageK - 1) / kStageK;
   const int chunks = (stages_total + kStages - 1) / kStages;
+  // K split over workgroups: this one multiplies chunks [chunk_begin, chunk_end) and writes to its own slice of d
+  const int chunk_begin = blockIdx.y * p.chunks_per_split;  // the launcher makes every split non-empty
+  const int chunk_end = chunk_begin + p.chunks_per_split < chunks ? chunk_begin + p.chunks_per_split : chunks;
+  char* const d_out = reinterpret_cast<char*>(p.d) + (size_t)blockIdx.y * p.m * p.n * (p.d_f16 ? 2 : 4);
 
   if constexpr (DMA) {
     // ---- asynchronous copy pattern for B: NL 16-byte copies per thread per stage ----
@@ -413,10 +417,11 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
       copy_row[i] = row;
       lds_dst[i] = smem_base + (NW * i + wave) * 1024;
     }
-    const char* b_stage = reinterpret_cast<const char*>(p.b) + (size_t)n0 * 2;  // advances one stage per copy
     const size_t stage_stride = (size_t)kStageK * p.n * 2;
+    const char* b_stage = reinterpret_cast<const char*>(p.b) + (size_t)n0 * 2 +
+                          (size_t)chunk_begin * kStages * stage_stride;  // advances one stage per copy
     const char* zeros = reinterpret_cast<const char*>(g_zero16);
-    int next_k0 = 0;  // first K row of the next stage to copy
+    int next_k0 = chunk_begin * kChunkK;  // first K row of the next stage to copy
     // Rows at or past K are copied from a block of zeros, so stages past the end of K (the ring always runs
     // whole chunks of four stages) and the padding of the prepared operand contribute nothing, and the
     // number of copies in flight, which the vmcnt waits rely on, is the same in every iteration.
@@ -460,8 +465,8 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
         a_dst[j] = smem_base + TS::LDS_B_BYTES + (NW * j + wave) * 1024;
       }
     }
-    const char* a_chunk = reinterpret_cast<const char*>(p.prep);  // advances one K chunk per copy
-    int next_chunk = 0;
+    const char* a_chunk = reinterpret_cast<const char*>(p.prep) + (size_t)chunk_begin * kBlockBytes;  // advances one K chunk per copy
+    int next_chunk = chunk_begin;
     auto issue_a = [&]() {
       if (ONEBIT_EXP_NO_COPY || ONEBIT_EXP_COPY_MODE == 1) return;
 #pragma unroll
@@ -507,7 +512,7 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
       load_b_frags<FN, BN>(smem + (((S) + 1) % kStages) * TS::STAGE_BYTES, 0, bv0, frag_off, lane_row_off);       \
     }
 
-    for (int kc = 0; kc < chunks; ++kc) {
+    for (int kc = chunk_begin; kc < chunk_end; ++kc) {
       // mid stage 0: waits for B(4c+1); newer requests: B(4c+2), B(4c+3)
       ONEBIT_STAGE(0, 2 * NL, true)
       expand_frags<2>(a_cur, one, av0);
@@ -544,7 +549,7 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
     wait_vmcnt<0>();  // drain the copies issued past the end before the LDS is released
   } else {
     // ---- generic path: any N, any K % 32 == 0, any alignment. One stage at a time, element copies. ----
-    for (int kc = 0; kc < chunks; ++kc) {
+    for (int kc = chunk_begin; kc < chunk_end; ++kc) {
       AChunk a_cur[FM];
 #pragma unroll
       for (int fm = 0; fm < FM; ++fm) a_cur[fm] = load_a_chunk(a_block[fm] + (size_t)kc * kBlockBytes, lane);
@@ -616,7 +621,7 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
               half8_t out;
 #pragma unroll
               for (int j = 0; j < 8; ++j) out[j] = (_Float16)x[j];
-              *reinterpret_cast<half8_t*>(reinterpret_cast<_Float16*>(p.d) + o) = out;
+              *reinterpret_cast<half8_t*>(reinterpret_cast<_Float16*>(d_out) + o) = out;
             }
           }
         } else {
@@ -644,7 +649,7 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
                   for (int j = 0; j < 4; ++j) x[j] = x[j] + p.beta * cv[j];
                 }
               }
-              *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.d) + o) = float4{x[0], x[1], x[2], x[3]};
+              *reinterpret_cast<float4*>(reinterpret_cast<float*>(d_out) + o) = float4{x[0], x[1], x[2], x[3]};
             }
           }
         }
@@ -671,8 +676,8 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
                                      : reinterpret_cast<const float*>(p.c)[o];
             x = x + p.beta * cv;
           }
-          if (p.d_f16) reinterpret_cast<_Float16*>(p.d)[o] = (_Float16)x;
-          else reinterpret_cast<float*>(p.d)[o] = x;
+          if (p.d_f16) reinterpret_cast<_Float16*>(d_out)[o] = (_Float16)x;
+          else reinterpret_cast<float*>(d_out)[o] = x;
         }
       }
     }
@@ -904,6 +909,52 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
 }
 
 // =====================================================================================================
+// splitk_reduce_kernel: d = alpha * (sum over splits, in split order, of the fp32 partial sums) + beta * c.
+// Elementwise over the m * n results; VEC = 4 when the element count and the alignment of c and d allow it.
+// =====================================================================================================
+template <int VEC>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, int splits, size_t stride,
+                                                            const void* __restrict__ c, void* __restrict__ d,
+                                                            size_t total, float alpha, float beta, int c_f16,
+                                                            int d_f16) {
+  const size_t first = ((size_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+  if (first >= total) return;
+  float x[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) x[j] = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float* src = ws + (size_t)s * stride + first;
+    if (VEC == 4) {
+      const float4 v = *reinterpret_cast<const float4*>(src);
+      x[0] += v.x; x[1 % VEC] += v.y; x[2 % VEC] += v.z; x[3 % VEC] += v.w;
+    } else {
+      x[0] += src[0];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    x[j] = alpha * x[j];
+    if (beta != 0.f) {
+      const float cv = c_f16 ? (float)reinterpret_cast<const _Float16*>(c)[first + j]
+                             : reinterpret_cast<const float*>(c)[first + j];
+      x[j] = x[j] + beta * cv;
+    }
+  }
+  if (VEC == 4) {
+    if (d_f16) {
+      typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+      *reinterpret_cast<half4_t*>(reinterpret_cast<_Float16*>(d) + first) =
+          half4_t{(_Float16)x[0], (_Float16)x[1 % VEC], (_Float16)x[2 % VEC], (_Float16)x[3 % VEC]};
+    } else {
+      *reinterpret_cast<float4*>(reinterpret_cast<float*>(d) + first) = float4{x[0], x[1 % VEC], x[2 % VEC], x[3 % VEC]};
+    }
+  } else {
+    if (d_f16) reinterpret_cast<_Float16*>(d)[first] = (_Float16)x[0];
+    else reinterpret_cast<float*>(d)[first] = x[0];
+  }
+}
+
+// =====================================================================================================
 // Host-side launchers
 // =====================================================================================================
 hipError_t launch_prepare(const void* a, const void* e, void* prep, int m, int k, int layout, hipStream_t stream) {
@@ -939,12 +990,11 @@ static hipError_t launch_gemm_cfg(GemmArgs args, hipStream_t stream) {
     if (st != hipSuccess) return st;
     attr_done[device] = true;
   }
-  hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n), dim3(64 * TS::NW), lds, stream, args);
+  hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, args.splits), dim3(64 * TS::NW), lds, stream, args);
   return hipGetLastError();
 }
 
-hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
-  if (prepared_bytes(args.m, args.k) >= (size_t(1) << 32)) return hipErrorInvalidValue;  // 32-bit copy offsets
+static hipError_t launch_gemm_pass(GemmArgs args, int tile_config, hipStream_t stream) {
   const bool aligned = (args.n % 8 == 0) && ((reinterpret_cast<uintptr_t>(args.b) & 15) == 0);
   // the coalesced epilogue moves 16 bytes per lane: n % 8 == 0 keeps every row start aligned when the bases are
   args.vector_epilogue = (reinterpret_cast<uintptr_t>(args.d) & 15) == 0 &&
@@ -963,6 +1013,38 @@ hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
     case kTile512x128w8: return launch_gemm_cfg<4, 2, 4, 2, true>(args, stream);
     default: return hipErrorInvalidValue;
   }
+}
+
+hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
+  if (prepared_bytes(args.m, args.k) >= (size_t(1) << 32)) return hipErrorInvalidValue;  // 32-bit copy offsets
+  const int chunks = (args.k + kChunkK - 1) / kChunkK;
+  if (args.splits <= 1) {
+    args.splits = 1;
+    args.chunks_per_split = chunks;
+    return launch_gemm_pass(args, tile_config, stream);
+  }
+  if (args.chunks_per_split < 1 || (long)(args.splits - 1) * args.chunks_per_split >= chunks || !args.split_ws)
+    return hipErrorInvalidValue;  // an empty split would address past the prepared operand
+  // pass 1: raw fp32 partial sums per split; pass 2: ordered sum and epilogue
+  GemmArgs pass = args;
+  pass.alpha = 1.f;
+  pass.beta = 0.f;
+  pass.c = nullptr;
+  pass.d = args.split_ws;
+  pass.d_f16 = 0;
+  if (hipError_t st = launch_gemm_pass(pass, tile_config, stream); st != hipSuccess) return st;
+  const size_t total = (size_t)args.m * args.n;
+  const bool vec = total % 4 == 0 && (reinterpret_cast<uintptr_t>(args.d) & 15) == 0 &&
+                   (args.beta == 0.f || (reinterpret_cast<uintptr_t>(args.c) & 15) == 0);
+  if (vec)
+    hipLaunchKernelGGL(splitk_reduce_kernel<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream,
+                       args.split_ws, args.splits, total, args.c, args.d, total, args.alpha, args.beta, args.c_f16,
+                       args.d_f16);
+  else
+    hipLaunchKernelGGL(splitk_reduce_kernel<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                       args.split_ws, args.splits, total, args.c, args.d, total, args.alpha, args.beta, args.c_f16,
+                       args.d_f16);
+  return hipGetLastError();
 }
 
 template <int NW, int R, int MODE>

@@ -16,6 +16,12 @@ struct GemmArgs {
   int c_f16, d_f16;      // 1: fp16, 0: fp32
   int tiles_m, tiles_n;  // filled by the launcher
   int vector_epilogue;   // filled by the launcher: C and D allow 16-byte accesses
+  // K split over workgroups (grid.y = splits): split s multiplies the K chunks [s * chunks_per_split, +chunks_per_split)
+  // and writes raw fp32 sums to split_ws + s * m * n; a second kernel adds the splits in order and applies the
+  // epilogue. splits <= 1: one pass straight into d. split_ws: at least splits * m * n floats, 16-byte aligned.
+  int splits;
+  int chunks_per_split;
+  float* split_ws;
 };
 
 struct SkinnyArgs {

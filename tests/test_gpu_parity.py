@@ -25,10 +25,12 @@ def _defaults():
     _native.set_tile_config(-1)
     _native.set_skinny_enabled(True)
     _native.set_skinny_rows(-1)
+    _native.set_split_k(-1)
     yield
     _native.set_tile_config(-1)
     _native.set_skinny_enabled(True)
     _native.set_skinny_rows(-1)
+    _native.set_split_k(-1)
 
 
 def _gpu(*ts):
@@ -205,6 +207,45 @@ def test_split_k_workgroup_shapes(rows, m, n, k):
     assert np.array_equal(got, exact)
     b = synthetic.make_b(k, n, seed=n + 50, kind="normal")
     _assert_close(_run_prepared(a, meta, b, m, n, k), oracle.blas_matmul(dense, b.numpy()))
+
+
+@pytest.mark.parametrize("splits", [-1, 1, 2, 3, 16])
+@pytest.mark.parametrize("m,n,k", [(256, 128, 4096), (192, 40, 2080), (1024, 264, 1024), (128, 1000, 4128)])
+def test_k_split_over_workgroups(splits, m, n, k):
+    """main kernel with K split over workgroups (partial sums + ordered reduction): forced split counts that do and
+    do not divide the chunk count, K tails, ragged N (generic variant), beta != 0, fp16 and fp32 results"""
+    _native.set_split_k(splits)
+    a, meta = synthetic.make_weight(m, k, seed=splits + m + k)
+    dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
+    bi = synthetic.make_b(k, n, seed=n, kind="int")
+    ci = synthetic.make_c(m, n, seed=n + 1, dtype=torch.float32).round()
+    exact = oracle.host_gemm(dense, bi.numpy(), c=ci.numpy(), alpha=2.0, beta=1.0, d_dtype=oracle.F32, acc="f32")
+    got = _run_prepared(a, meta, bi, m, n, k, c=ci, alpha=2.0, beta=1.0, out_dtype=torch.float32)
+    assert np.array_equal(got, exact)
+    exact16 = oracle.host_gemm(dense, bi.numpy(), d_dtype=oracle.F16, acc="f32")
+    assert np.array_equal(_run_prepared(a, meta, bi, m, n, k, out_dtype=torch.float16), exact16)
+    b = synthetic.make_b(k, n, seed=n + 50, kind="normal")
+    _assert_close(_run_prepared(a, meta, b, m, n, k), oracle.blas_matmul(dense, b.numpy()))
+
+
+def test_k_split_streams_do_not_share_partial_sums():
+    m, n, k = 256, 128, 8192
+    a, meta = synthetic.make_weight(m, k, seed=9)
+    ad, md = _gpu(a, meta)
+    prep = _native.prepare(ad, md, m, k)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    bs = [synthetic.make_b(k, n, seed=20 + i, kind="int").cuda() for i in range(3)]
+    outs = [torch.empty((m, n), dtype=torch.float32, device="cuda") for _ in range(3)]
+    torch.cuda.synchronize()
+    for _ in range(20):
+        for s, b, o in zip(streams, bs, outs):
+            with torch.cuda.stream(s):
+                _native.matmul_prepared(prep, b, o, m, n, k)
+    torch.cuda.synchronize()
+    dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
+    for b, o in zip(bs, outs):
+        assert np.array_equal(o.cpu().numpy(), oracle.host_gemm(dense, b.cpu().numpy(), d_dtype=oracle.F32, acc="f32"))
 
 
 def test_config3_split_k_is_deterministic_and_reusable():
