@@ -146,7 +146,7 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
     int rows = g_skinny_rows.load();
     // the largest row group that still gives about two workgroups per three compute units (measured: larger groups
     // re-read B less often, but idle compute units cost more)
-    if (rows <= 0) rows = (m / 128 >= 160) ? 128 : (m / 64 >= 160) ? 64 : 32;
+    if (rows <= 0) rows = (m / 128 >= 160 && n <= 16) ? 128 : (m / 64 >= 160) ? 64 : 32;
     ONEBIT_HIP(onebit::launch_skinny(args, rows, stream));
     return ONEBIT_OK;
   }

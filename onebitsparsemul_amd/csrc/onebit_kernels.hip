@@ -685,39 +685,42 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
 }
 
 // =====================================================================================================
-// skinny_kernel: N <= 16 (decode shapes). HBM-bound: every byte of the prepared operand is read once.
+// skinny_kernel: N <= 32 (decode shapes). HBM-bound: every byte of the prepared operand is read once.
 // Workgroup = NW wavefronts that share R row blocks (32 rows each) and split K among themselves: wavefront w
-// takes the K chunks (of 256) w, w + NW, w + 2 NW, ... Each wavefront stages the B rows of its chunk in a private
-// 8 KiB LDS region as a zero-padded [256][16] fp16 image, feeds them to SMFMAC through transpose reads (one
-// fragment serves the R row blocks) and keeps a 32x32 fp32 partial tile per row block. The prepared operand and
-// the B rows of the wavefront's next chunk are loaded into registers while the current chunk is multiplied.
-// Wavefronts never wait for one another inside the K loop (LDS operations of one wavefront execute in order).
-// The NW partial tiles of a row block are added through LDS in wavefront order (deterministic) and the epilogue
-// is applied. grid = M / (32 R) workgroups; no global workspace, no atomics.
+// takes the K chunks (of 256) w, w + NW, w + 2 NW, ... Each wavefront stages B rows in a private 8 KiB LDS region
+// as a zero-padded fp16 image of NC columns (NC = 16: the 256 rows of a chunk; NC = 32: 128 rows, two images per
+// chunk), feeds them to SMFMAC through transpose reads (one fragment serves the R row blocks) and keeps a 32x32
+// fp32 partial tile per row block. The prepared operand and the next image are loaded into registers while the
+// current one is multiplied. Wavefronts never wait for one another inside the K loop (LDS operations of one
+// wavefront execute in order). The NW partial tiles of a row block are added through LDS in wavefront order
+// (deterministic) and the epilogue is applied. grid = M / (32 R) workgroups; no global workspace, no atomics.
 // =====================================================================================================
 #ifndef ONEBIT_EXP_SKINNY
 #define ONEBIT_EXP_SKINNY 0  // measurement builds (results wrong): 1 no B reloads, 2 one fragment group per chunk, 3 one expansion per chunk, 4 loads and image stores only
 #endif
-constexpr int kSkinnyRegion = kChunkK * 16 * 2;  // bytes of one B image
-constexpr int kSkinnyTileBytes = kRowBlock * 16 * 4;
+constexpr int kSkinnyRegion = 8192;  // bytes of one B image
 
-enum SkinnyBMode { kSkinnyB16 = 0, kSkinnyB8 = 1, kSkinnyB4 = 2, kSkinnyBScalar = 3 };
+// how B rows reach the image: whole rows are the image rows (n == NC), rows of n % 8 == 0 elements in 16-byte
+// pieces padded to the image row, 8-byte rows (n == 4, NC == 16), or element by element (any n <= NC, any alignment)
+enum SkinnyBMode { kSkinnyBFull = 0, kSkinnyB8 = 1, kSkinnyB4 = 2, kSkinnyBScalar = 3 };
 
-// 16-byte piece q of the image of the chunk at k_base: row q / 2, columns 8 (q % 2) ... + 7; zero outside B.
-// Vector modes only (n = 16, 8 or 4 with B aligned to its row size).
+// 16-byte piece q of the image whose first row is B row k_base: image row q / (NC / 8), columns 8 (q % (NC / 8))
+// ... + 7; zero outside B. Vector modes only.
+template <int NC>
 __device__ __forceinline__ u32x4_t skinny_load_piece(const _Float16* __restrict__ b, int n, int mode, int k_base,
                                                       int rows_valid, int q) {
-  const int row = q >> 1, h = q & 1;
+  constexpr int PPR = NC / 8;  // pieces per image row
+  const int row = q / PPR, h = q % PPR;
   const bool ok = row < rows_valid;
   const char* base = reinterpret_cast<const char*>(b);
   u32x4_t v = u32x4_t{0, 0, 0, 0};
-  if (mode == kSkinnyB16) {
-    const char* src = ok ? base + ((size_t)k_base * 16 + (size_t)q * 8) * 2 : base;
+  if (mode == kSkinnyBFull) {
+    const char* src = ok ? base + ((size_t)k_base * NC + (size_t)q * 8) * 2 : base;
     v = *reinterpret_cast<const u32x4_t*>(src);
     if (!ok) v = u32x4_t{0, 0, 0, 0};
   } else if (mode == kSkinnyB8) {
-    const bool use = ok && h == 0;
-    const char* src = use ? base + (size_t)(k_base + row) * 16 : base;
+    const bool use = ok && 8 * h < n;
+    const char* src = use ? base + ((size_t)(k_base + row) * n + 8 * h) * 2 : base;
     v = *reinterpret_cast<const u32x4_t*>(src);
     if (!use) v = u32x4_t{0, 0, 0, 0};
   } else {  // kSkinnyB4
@@ -729,10 +732,17 @@ __device__ __forceinline__ u32x4_t skinny_load_piece(const _Float16* __restrict_
   return v;
 }
 
-template <int NW, int R, int MODE>
+template <int NW, int R, int MODE, int NC>
 __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(SkinnyArgs p) {
   constexpr int NT = 64 * NW;
-  static_assert(R * kSkinnyTileBytes <= kSkinnyRegion, "partial tiles reuse the wavefront's image memory");
+  constexpr int IMG_ROWS = kSkinnyRegion / (NC * 2);   // B rows per image: 256 or 128
+  constexpr int SUB = kChunkK / IMG_ROWS;              // images per chunk: 1 or 2
+  constexpr int IMG_STEPS = kStepsPerChunk / SUB;      // 32-wide K steps per image: 8 or 4
+  constexpr int ROW_BYTES = NC * 2;
+  constexpr int TILE_BYTES = kRowBlock * NC * 4;       // one fp32 partial tile
+  static_assert(NC == 16 || NC == 32, "image width");
+  static_assert(MODE != kSkinnyB4 || NC == 16, "the 8-byte-row mode is for 16 columns");
+  static_assert(R * TILE_BYTES <= kSkinnyRegion, "partial tiles reuse the wavefront's image memory");
   __shared__ __attribute__((aligned(16))) char bs[NW * kSkinnyRegion];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -755,36 +765,50 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   };
   auto rows_valid_of = [&](int k_base) __attribute__((always_inline)) {
     const int rows = k_rows - k_base;
-    return rows < 0 ? 0 : (rows > kChunkK ? kChunkK : rows);
+    return rows < 0 ? 0 : (rows > IMG_ROWS ? IMG_ROWS : rows);
   };
-  // vector modes: the image of a chunk travels through registers, loaded while the previous chunk is multiplied;
-  // element mode (any n, any alignment): loaded and stored in one go when the image is due, piece by piece
-  auto load_b = [&](int kc, u32x4_t (&v)[8]) __attribute__((always_inline)) {
+  // element mode: image position of element `lane` of an image's run of IMG_ROWS * n elements, and the step of 64
+  const int elem_col0 = lane % n_cols;
+  const int elem_offset0 = (lane / n_cols) * ROW_BYTES + elem_col0 * 2;
+  const int step_cols = 64 % n_cols;
+  const int step_bytes = (64 / n_cols) * ROW_BYTES + step_cols * 2;
+  // Image t of this wavefront = B rows [k_base, k_base + IMG_ROWS) with k_base = (wave + NW (t / SUB)) * 256 +
+  // (t % SUB) * IMG_ROWS. Vector modes: the image travels through registers, loaded while the previous image is
+  // multiplied; element mode: loaded and stored in one go when the image is due.
+  auto load_b = [&](int k_base, u32x4_t (&v)[8]) __attribute__((always_inline)) {
     if (MODE == kSkinnyBScalar) return;
-    const int k_base = kc * kChunkK;
     const int rows_valid = rows_valid_of(k_base);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = skinny_load_piece(b_ptr, n_cols, MODE, k_base, rows_valid, lane + i * 64);
+    for (int i = 0; i < 8; ++i) v[i] = skinny_load_piece<NC>(b_ptr, n_cols, MODE, k_base, rows_valid, lane + i * 64);
   };
-  auto store_b = [&](int kc, const u32x4_t (&v)[8]) __attribute__((always_inline)) {
+  auto store_b = [&](int k_base, const u32x4_t (&v)[8]) __attribute__((always_inline)) {
     if (MODE == kSkinnyBScalar) {
-      // the chunk's rows are one run of 256 n elements; rows at or past K are written as zeros, the padding
-      // columns n ... 15 keep the zeros the image was cleared to
-      const int k_base = kc * kChunkK;
-      const int valid = rows_valid_of(k_base) * n_cols, total = kChunkK * n_cols;
+      // the image's rows are one run of IMG_ROWS n elements; rows at or past K are written as zeros, the padding
+      // columns n ... NC - 1 keep the zeros the image was cleared to
+      const int valid = rows_valid_of(k_base) * n_cols, total = IMG_ROWS * n_cols;
       const _Float16* src = b_ptr + (size_t)k_base * n_cols;
-      for (int e0 = lane; e0 < total; e0 += 64 * 4) {
-        uint16_t bits[4];
+      constexpr int BATCH = NC == 32 ? 16 : 4;  // loads in flight per lane
+      int offset = elem_offset0;  // byte offset in the image of element e = lane + 64 i, kept without divisions
+      int col = elem_col0;
+      for (int e0 = lane; e0 < total; e0 += 64 * BATCH) {
+        uint16_t bits[BATCH];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < BATCH; ++i) {
           const int e = e0 + i * 64;
           bits[i] = __builtin_bit_cast(uint16_t, e < valid ? src[e] : b_ptr[0]);
           if (e >= valid) bits[i] = 0;
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < BATCH; ++i) {
           const int e = e0 + i * 64;
-          if (e < total) *reinterpret_cast<uint16_t*>(region + (e / n_cols) * 32 + (e % n_cols) * 2) = bits[i];
+          if (e < total) *reinterpret_cast<uint16_t*>(region + offset) = bits[i];
+          // e += 64: 64 / n rows further and 64 % n columns, with one carry at most
+          col += step_cols;
+          offset += step_bytes;
+          if (col >= n_cols) {
+            col -= n_cols;
+            offset += ROW_BYTES - n_cols * 2;
+          }
         }
       }
       return;
@@ -800,21 +824,24 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
     for (int v = 0; v < 16; ++v) acc[r][v] = 0.f;
   const uint32_t one = packed_one_in_vgpr();
   const int i16 = lane & 15, gb = lane >> 5;
-  // lanes 16-31 and 48-63 would hold columns 16-31: they re-read columns 0-15 and are never stored
-  const char* lane_ptr = region + (8 * gb + (i16 >> 2)) * 32 + (i16 & 3) * 8;
+  // NC == 16: lanes 16-31 and 48-63 would hold columns 16-31: they re-read columns 0-15 and are never stored
+  const int chunk8 = (NC == 32 ? ((lane & 31) >> 4) * 4 : 0) + (i16 & 3);  // 8-byte piece of the image row
+  const char* lane_ptr = region + (8 * gb + (i16 >> 2)) * ROW_BYTES + chunk8 * 8;
 
-  auto frag = [&](int st) __attribute__((always_inline)) {
+  auto frag = [&](int image_step) __attribute__((always_inline)) {
     u32x8_t raw;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const int row_const = st * 32 + 4 * (q & 1) + 16 * (q >> 1);
-      const u32x2_t t = lds_read_tr16(lane_ptr + row_const * 32);
+      const int row_const = image_step * 32 + 4 * (q & 1) + 16 * (q >> 1);
+      const u32x2_t t = lds_read_tr16(lane_ptr + row_const * ROW_BYTES);
       raw[2 * q] = t.x;
       raw[2 * q + 1] = t.y;
     }
     return __builtin_bit_cast(half16_t, raw);
   };
-  auto compute = [&](const AChunk (&a)[R]) __attribute__((always_inline)) {
+  // the SMFMACs of image SUB_INDEX of a chunk: steps SUB_INDEX * IMG_STEPS ... + IMG_STEPS - 1
+  auto compute = [&](const AChunk (&a)[R], auto sub_tag) __attribute__((always_inline)) {
+    constexpr int FIRST_STEP = decltype(sub_tag)::value * IMG_STEPS;
     // FG fragments (4 FG transpose reads) in flight, then their SMFMACs back to back; the scheduling barriers keep
     // the next group's reads from being hoisted (8 registers per fragment)
     constexpr int FG = R >= 4 ? 2 : 4;
@@ -830,71 +857,85 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
 #endif
     };
     auto group = [&](auto first_tag) __attribute__((always_inline)) {
-      constexpr int FIRST = decltype(first_tag)::value;
+      constexpr int FIRST = decltype(first_tag)::value;  // step within the chunk
 #if ONEBIT_EXP_SKINNY == 2
       if (FIRST == 0)
 #endif
 #pragma unroll
-      for (int st = 0; st < FG; ++st) bfrag[st] = frag(FIRST + st);
+      for (int st = 0; st < FG; ++st) bfrag[st] = frag(FIRST - FIRST_STEP + st);
       step(std::integral_constant<int, FIRST>{});
       step(std::integral_constant<int, FIRST + 1>{});
       if constexpr (FG == 4) {
         step(std::integral_constant<int, FIRST + 2>{});
         step(std::integral_constant<int, FIRST + 3>{});
       }
-      if (FIRST + FG < kStepsPerChunk) __builtin_amdgcn_sched_barrier(0);
+      if (FIRST + FG < FIRST_STEP + IMG_STEPS) __builtin_amdgcn_sched_barrier(0);
     };
-    group(std::integral_constant<int, 0>{});
-    if constexpr (FG == 2) group(std::integral_constant<int, 2>{});
-    group(std::integral_constant<int, 4>{});
-    if constexpr (FG == 2) group(std::integral_constant<int, 6>{});
+    group(std::integral_constant<int, FIRST_STEP>{});
+    if constexpr (IMG_STEPS > FG) group(std::integral_constant<int, FIRST_STEP + FG>{});
+    if constexpr (IMG_STEPS > 2 * FG) group(std::integral_constant<int, FIRST_STEP + 2 * FG>{});
+    if constexpr (IMG_STEPS > 3 * FG) group(std::integral_constant<int, FIRST_STEP + 3 * FG>{});
   };
 
   // sixteen wavefronts leave 128 registers each: no room to hold the next image (32 registers) during the SMFMACs
   constexpr bool kPrefetchB = NW <= 8 && MODE != kSkinnyBScalar;
+  if (MODE == kSkinnyBScalar) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4_t*>(region + (lane + i * 64) * 16) = u32x4_t{0, 0, 0, 0};
+  }
   u32x4_t breg[8];
   AChunk a_cur[R], a_next[R];
-  if (kPrefetchB) load_b(wave, breg);
+  if (kPrefetchB) load_b(wave * kChunkK, breg);
   load_a(wave, a_cur);
   for (int kc = wave; kc < kc_total; kc += NW) {
-    if (!kPrefetchB) load_b(kc, breg);
-    store_b(kc, breg);  // after the previous chunk's fragment reads: LDS operations of a wavefront execute in order
+    const int k_base = kc * kChunkK;
+    if (!kPrefetchB) load_b(k_base, breg);
+    store_b(k_base, breg);  // after the previous image's fragment reads: LDS operations of a wavefront execute in order
 #if ONEBIT_EXP_SKINNY != 1
-    if (kPrefetchB) load_b(kc + NW, breg);
+    if (kPrefetchB) load_b(SUB == 2 ? k_base + IMG_ROWS : k_base + NW * kChunkK, breg);
 #endif
     load_a(kc + NW, a_next);
 #if ONEBIT_EXP_SKINNY == 4
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r][0] += __builtin_bit_cast(float, a_cur[r].meta.x ^ a_cur[r].sign.y);
 #else
-    compute(a_cur);
+    compute(a_cur, std::integral_constant<int, 0>{});
+    if constexpr (SUB == 2) {
+      if (!kPrefetchB) {
+        __builtin_amdgcn_sched_barrier(0);  // the second image's loads stay behind the first image's SMFMACs
+        load_b(k_base + IMG_ROWS, breg);
+      }
+      store_b(k_base + IMG_ROWS, breg);
+      if (kPrefetchB) load_b(k_base + NW * kChunkK, breg);
+      compute(a_cur, std::integral_constant<int, 1>{});
+    }
 #endif
 #pragma unroll
     for (int r = 0; r < R; ++r) a_cur[r] = a_next[r];
   }
 
   smfmac_drain();
-  // ---- add the NW partial tiles through LDS: region of wavefront w := its R tiles as [r][32 rows][16 cols] fp32
+  // ---- add the NW partial tiles through LDS: region of wavefront w := its R tiles as [r][32 rows][NC cols] fp32
   {
     float* tile = reinterpret_cast<float*>(region);
     const int col = lane & 31;
-    if (col < 16) {
+    if (col < NC) {
 #pragma unroll
       for (int r = 0; r < R; ++r)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int row = 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-          tile[(r * 32 + row) * 16 + col] = acc[r][v];
+          tile[(r * 32 + row) * NC + col] = acc[r][v];
         }
     }
   }
   __syncthreads();
-  for (int idx = tid; idx < R * kRowBlock * 16; idx += NT) {
+  for (int idx = tid; idx < R * kRowBlock * NC; idx += NT) {
     float sum = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) sum += reinterpret_cast<const float*>(bs + w * kSkinnyRegion)[idx];
-    const int col = idx & 15;
-    const int row = rb_first * kRowBlock + (idx >> 4);
+    const int col = idx % NC;
+    const int row = rb_first * kRowBlock + idx / NC;
     if (col < p.n && row < p.m) {
       const size_t o = (size_t)row * p.n + col;
       float x = p.alpha * sum;
@@ -1047,27 +1088,34 @@ hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <int NW, int R, int MODE>
+template <int NW, int R, int MODE, int NC>
 static hipError_t launch_skinny_mode(const SkinnyArgs& args, hipStream_t stream) {
   const int row_blocks = args.m / kRowBlock;
-  hipLaunchKernelGGL((skinny_kernel<NW, R, MODE>), dim3((row_blocks + R - 1) / R), dim3(64 * NW), 0, stream, args);
+  hipLaunchKernelGGL((skinny_kernel<NW, R, MODE, NC>), dim3((row_blocks + R - 1) / R), dim3(64 * NW), 0, stream, args);
   return hipGetLastError();
 }
 
 template <int NW, int R>
 static hipError_t launch_skinny_cfg(const SkinnyArgs& args, hipStream_t stream) {
   const uintptr_t address = reinterpret_cast<uintptr_t>(args.b);
-  if (args.n == 16 && (address & 15) == 0) return launch_skinny_mode<NW, R, kSkinnyB16>(args, stream);
-  if (args.n == 8 && (address & 15) == 0) return launch_skinny_mode<NW, R, kSkinnyB8>(args, stream);
-  if (args.n == 4 && (address & 7) == 0) return launch_skinny_mode<NW, R, kSkinnyB4>(args, stream);
-  return launch_skinny_mode<NW, R, kSkinnyBScalar>(args, stream);
+  if (args.n > 16) {  // 32-column images; their two partial tiles per row block fill the image memory at R = 2
+    constexpr int R32 = R > 2 ? 2 : R;
+    if (args.n == 32 && (address & 15) == 0) return launch_skinny_mode<NW, R32, kSkinnyBFull, 32>(args, stream);
+    if (args.n % 8 == 0 && (address & 15) == 0) return launch_skinny_mode<NW, R32, kSkinnyB8, 32>(args, stream);
+    return launch_skinny_mode<NW, R32, kSkinnyBScalar, 32>(args, stream);
+  }
+  if (args.n == 16 && (address & 15) == 0) return launch_skinny_mode<NW, R, kSkinnyBFull, 16>(args, stream);
+  if (args.n == 8 && (address & 15) == 0) return launch_skinny_mode<NW, R, kSkinnyB8, 16>(args, stream);
+  if (args.n == 4 && (address & 7) == 0) return launch_skinny_mode<NW, R, kSkinnyB4, 16>(args, stream);
+  return launch_skinny_mode<NW, R, kSkinnyBScalar, 16>(args, stream);
 }
 
 hipError_t launch_skinny(SkinnyArgs args, int rows_per_group, hipStream_t stream) {
+  if (args.n < 1 || args.n > kSkinnyMaxN) return hipErrorInvalidValue;
   switch (rows_per_group) {
     case 32: return launch_skinny_cfg<16, 1>(args, stream);  // sixteen wavefronts split K: small M
     case 64: return launch_skinny_cfg<8, 2>(args, stream);
-    case 128: return launch_skinny_cfg<8, 4>(args, stream);
+    case 128: return launch_skinny_cfg<8, 4>(args, stream);  // n > 16: 64-row groups
     default: return hipErrorInvalidValue;
   }
 }

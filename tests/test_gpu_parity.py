@@ -193,10 +193,12 @@ def test_config3_decode(m, k, n):
 
 @pytest.mark.parametrize("rows", [32, 64, 128])
 @pytest.mark.parametrize("m,n,k", [(64, 1, 32), (192, 5, 800), (320, 8, 4128), (4096, 16, 4096), (1088, 4, 2048),
-                                   (2240, 16, 8224), (128, 13, 12320)])
+                                   (2240, 16, 8224), (128, 13, 12320), (192, 32, 800), (4096, 32, 4096),
+                                   (320, 17, 4128), (1088, 31, 2208), (64, 24, 32)])
 def test_split_k_workgroup_shapes(rows, m, n, k):
     """every row-group size of the split-K kernel: chunk counts that do not divide among the wavefronts, a row
-    group past the last row block, K tails, every B staging mode (n = 16, 8, 4 vector copies; element copies)"""
+    group past the last row block, K tails, every B staging mode (n = 32, 16, 8, 4 vector copies; element
+    copies), 16- and 32-column images"""
     _native.set_skinny_rows(rows)
     a, meta = synthetic.make_weight(m, k, seed=rows + m + k)
     dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
@@ -325,8 +327,9 @@ def test_every_tile_configuration(tile, m, n, k):
     assert np.array_equal(got, exact)
 
 
-def test_unaligned_b_pointer():
-    m, n, k = 256, 64, 128
+@pytest.mark.parametrize("n", [64, 32, 16, 8])  # main kernel's element-copy variant; split-K kernel's element mode
+def test_unaligned_b_pointer(n):
+    m, k = 256, 128
     a, meta = synthetic.make_weight(m, k, seed=9)
     bi = synthetic.make_b(k, n, seed=9, kind="int")
     exact = oracle.reference_matmul(a.numpy(), bi.numpy(), meta.numpy(), m, n, k, d_dtype=oracle.F32)
