@@ -24,39 +24,53 @@ __global__ __launch_bounds__(64) void prepare_kernel(const uint8_t* __restrict__
                                                      int layout) {
   const int kc = blockIdx.x, rb = blockIdx.y, lane = threadIdx.x;
   const int i = lane & 31, ga = lane >> 5;
-  const int64_t r = (int64_t)rb * kRowBlock + i;
+  const int64_t r = (int64_t)rb * kRowBlock + i;  // m % 32 == 0: every row of the block exists
   const int ncols = k / 16;
+  // The value bits of the block's 32 rows for one compressed column are one aligned dword of `a` (bit position
+  // 32 rb + j m, m % 32 == 0). The block spans 128 compressed columns: two dwords per lane, shared through LDS.
+  __shared__ __attribute__((aligned(16))) uint32_t column_bits[128];
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    const int local = lane + 64 * half;
+    const int64_t j = (int64_t)kc * 128 + local;     // compressed column
+    uint32_t word = 0xFFFFFFFFu;                      // padding past K: +1
+    if (j < k / 2) {
+      const uint8_t* src = a + (((int64_t)rb * kRowBlock + j * m) >> 3);
+      if ((reinterpret_cast<uintptr_t>(a) & 3) == 0)
+        word = *reinterpret_cast<const uint32_t*>(src);
+      else
+        word = (uint32_t)src[0] | ((uint32_t)src[1] << 8) | ((uint32_t)src[2] << 16) | ((uint32_t)src[3] << 24);
+    }
+    column_bits[local] = word;
+  }
+  __syncthreads();
   uint32_t meta[4] = {0, 0, 0, 0};
   uint32_t sign[2] = {0, 0};
-  if (r < m) {
 #pragma unroll
-    for (int s = 0; s < kStepsPerChunk; ++s) {
-      const int c = kc * 16 + 2 * s + ga;
-      uint32_t mv = 0x4444u;
-      uint32_t neg = 0;  // bit t set: kept value t of this step is -1
-      if (c < ncols) {
-        int64_t off;
-        if (layout == 0) off = meta_offset_reference(r, c, m);
-        else if (layout == 1) off = meta_offset_cutlass(r, c, m);
-        else off = r * ncols + c;
-        mv = e[off];
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-          const int64_t pos = r + (int64_t)(8 * c + t) * m;
-          const uint32_t bit = (a[pos >> 3] >> (pos & 7)) & 1u;
-          neg |= (bit ^ 1u) << t;
-        }
-      }
-      meta[s >> 1] |= mv << (16 * (s & 1));
-#pragma unroll
-      for (int p = 0; p < 4; ++p) {
-        const int j = 4 * (s & 3) + p;
-        sign[s >> 2] |= ((neg >> (2 * p)) & 1u) << (15 - j);
-        sign[s >> 2] |= ((neg >> (2 * p + 1)) & 1u) << (31 - j);
-      }
+  for (int s = 0; s < kStepsPerChunk; ++s) {
+    const int c = kc * 16 + 2 * s + ga;
+    uint32_t mv = 0x4444u;
+    if (c < ncols) {
+      int64_t off;
+      if (layout == 0) off = meta_offset_reference(r, c, m);
+      else if (layout == 1) off = meta_offset_cutlass(r, c, m);
+      else off = r * ncols + c;
+      mv = e[off];
     }
-  } else {
-    meta[0] = meta[1] = meta[2] = meta[3] = 0x44444444u;
+    meta[s >> 1] |= mv << (16 * (s & 1));
+    // kept value t of this step = compressed column 8 c + t = entry 8 (2 s + ga) + t of the block's 128
+    const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(&column_bits[8 * (2 * s + ga)]);
+    const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(&column_bits[8 * (2 * s + ga) + 4]);
+    const uint32_t w8[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    uint32_t neg = 0;  // bit t set: kept value t of this step is -1
+#pragma unroll
+    for (int t = 0; t < 8; ++t) neg |= (((w8[t] >> i) & 1u) ^ 1u) << t;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int j = 4 * (s & 3) + p;
+      sign[s >> 2] |= ((neg >> (2 * p)) & 1u) << (15 - j);
+      sign[s >> 2] |= ((neg >> (2 * p + 1)) & 1u) << (31 - j);
+    }
   }
   uint8_t* block = prep + ((size_t)rb * kc_total + kc) * kBlockBytes;
   u32x4_t mvec = {meta[0], meta[1], meta[2], meta[3]};

@@ -345,6 +345,22 @@ def test_unaligned_b_pointer(n):
     assert np.array_equal(d.cpu().numpy(), exact)
 
 
+def test_unaligned_value_bits_pointer():
+    """the one-bit operand at an address that is not a multiple of 4: the reorder kernel then reads it bytewise"""
+    m, n, k = 192, 48, 544
+    a, meta = synthetic.make_weight(m, k, seed=13)
+    bi = synthetic.make_b(k, n, seed=13, kind="int")
+    exact = oracle.reference_matmul(a.numpy(), bi.numpy(), meta.numpy(), m, n, k, d_dtype=oracle.F32)
+    storage = torch.zeros(a.numel() + 8, dtype=torch.uint8, device="cuda")
+    ad = storage[1:1 + a.numel()]
+    ad.copy_(a.cuda().reshape(-1))
+    assert ad.data_ptr() % 4 != 0
+    d = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    _native.matmul_ex(ad, bi.cuda(), meta.cuda(), d, m, n, k)
+    torch.cuda.synchronize()
+    assert np.array_equal(d.cpu().numpy(), exact)
+
+
 def test_reference_benchmark_dataset():
     """tests/kernel_test.cu:302-306,398-400: all value bits 1, all metadata 0x4444 => rows t % 4 < 2 of B summed."""
     m, n, k = 256, 128, 512
