@@ -186,16 +186,18 @@ struct TileShape {
 };
 
 // XCD-aware tile order. Workgroup b runs on XCD b % 8, so XCD x is given a contiguous range of a tile list
-// that is ordered in blocks of 16 row tiles x 4 column tiles (row tile fastest), blocks running down M inside a
-// strip of 4 column tiles, strips running along N. The ~64 workgroups resident on one XCD then form one block:
-// every B column panel it streams is shared by 16 workgroups and every A row panel by 4 in that XCD's L2, and
-// the whole range of one XCD covers few column strips, so B is fetched into few L2s.
+// that is ordered in blocks of GROUP_M row tiles x 4 column tiles (row tile fastest), blocks running down M inside
+// a strip of 4 column tiles, strips running along N. GROUP_M x 4 = the workgroups resident on one XCD (64 for the
+// four-wavefront tiles, two per CU; 32 for the eight-wavefront tiles), which then form one block: every B column
+// panel it streams is shared by GROUP_M workgroups and every A row panel by 4 in that XCD's L2, and the whole
+// range of one XCD covers few column strips, so B is fetched into few L2s.
+template <int GROUP_M>
 __device__ __forceinline__ void tile_of_block(int b, int tiles_m, int tiles_n, int& tm, int& tn) {
   const int total = tiles_m * tiles_n;
   const int per = total / 8, rem = total % 8;
   const int x = b % 8, local = b / 8;
   const int v = x * per + (x < rem ? x : rem) + local;
-  constexpr int GROUP_M = 16, STRIP_N = 4;
+  constexpr int STRIP_N = 4;
   const int strip = v / (tiles_m * STRIP_N);
   const int strip_w = (tiles_n - strip * STRIP_N) < STRIP_N ? (tiles_n - strip * STRIP_N) : STRIP_N;
   const int w = v - strip * STRIP_N * tiles_m;
@@ -256,6 +258,9 @@ __device__ __forceinline__ void compute_stage(const char* stage_lds, const AChun
 #endif
 #ifndef ONEBIT_EXP_WAIT_MODE  /* 1: never wait for copies (vmcnt 63), 2: always wait for all copies (vmcnt 0) */
 #define ONEBIT_EXP_WAIT_MODE 0
+#endif
+#ifndef ONEBIT_MAIN_ORDER    /* SMFMAC order inside a K step: 0 row fragments outer (A held), 1 column fragments outer (B held) */
+#define ONEBIT_MAIN_ORDER 0
 #endif
 #ifndef ONEBIT_MAIN_PINNED   /* 1: inline-asm SMFMAC with accumulators pinned to AGPRs where that fits, 0: builtin */
 #define ONEBIT_MAIN_PINNED 1
@@ -326,13 +331,21 @@ __device__ __forceinline__ void expand_frags(const AChunk (&a)[FM], uint32_t one
 template <int STEP, int FM, int FN>
 __device__ __forceinline__ void mfma_frags(const AChunk (&a)[FM], const half8_t (&av)[FM], const half16_t (&bv)[FN],
                                            float16_t (&acc)[FM][FN]) {
+  // pinned accumulators only for the one-wavefront-per-SIMD tiles: the two-per-SIMD tiles have 128 vector
+  // registers left beside their 128 accumulators, which the pinned form overflows
+#if ONEBIT_MAIN_ORDER == 1
+#pragma unroll
+  for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm)
+      acc[fm][fn] = smfmac_step<STEP, (ONEBIT_MAIN_PINNED != 0 && FM * FN > 8)>(a[fm], av[fm], bv[fn], acc[fm][fn]);
+#else
 #pragma unroll
   for (int fm = 0; fm < FM; ++fm)
 #pragma unroll
     for (int fn = 0; fn < FN; ++fn)
-      // pinned accumulators only for the one-wavefront-per-SIMD tiles: the two-per-SIMD tiles have 128 vector
-      // registers left beside their 128 accumulators, which the pinned form overflows
       acc[fm][fn] = smfmac_step<STEP, (ONEBIT_MAIN_PINNED != 0 && FM * FN > 8)>(a[fm], av[fm], bv[fn], acc[fm][fn]);
+#endif
 }
 
 // Pins the instruction order of one K-step region: each SMFMAC is followed by its share of the region's LDS
@@ -368,7 +381,7 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in a scalar register
   const int wm = wave / WN, wn = wave % WN;
   int tile_m, tile_n;
-  tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  tile_of_block<(NW == 8 ? 8 : 16)>(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
   const int row0 = tile_m * BM + wm * FM * 32;  // first row of this wavefront
   const int n0 = tile_n * BN;                   // first column of the workgroup
   const int col0 = n0 + wn * FN * 32;           // first column of this wavefront
