@@ -132,7 +132,10 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
   if (beta != 0.f && !c) return fail(ONEBIT_ERR_ARGUMENT, "c must not be null when beta != 0");
   const int kc_total = (k + onebit::kChunkK - 1) / onebit::kChunkK;
 
-  if (n <= onebit::kSkinnyMaxN && g_skinny_enabled.load()) {
+  // 32 < n <= 64: every 32-row workgroup of the split-K kernel stages all of B, which the main kernel's tiles
+  // overtake from about 16k rows on (28672 x 64 x 8192: 43 us against 58 us; 11008 x 64 x 4096: 21 against 17)
+  const bool skinny_shape = n <= 32 || (n <= onebit::kSkinnyMaxN && m <= 16384);
+  if (skinny_shape && g_skinny_enabled.load()) {
     onebit::SkinnyArgs args{};
     args.prep = static_cast<const uint8_t*>(prepared);
     args.b = static_cast<const _Float16*>(b);
@@ -146,7 +149,7 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
     int rows = g_skinny_rows.load();
     // the largest row group that still gives about two workgroups per three compute units (measured: larger groups
     // re-read B less often, but idle compute units cost more)
-    if (rows <= 0) rows = (m / 128 >= 160 && n <= 16) ? 128 : (m / 64 >= 160) ? 64 : 32;
+    if (rows <= 0) rows = n > 32 ? 32 : (m / 128 >= 160 && n <= 16) ? 128 : (m / 64 >= 160) ? 64 : 32;
     ONEBIT_HIP(onebit::launch_skinny(args, rows, stream));
     return ONEBIT_OK;
   }

@@ -1,7 +1,7 @@
 // gfx950 kernels of the one-bit 2:4 sparse GEMM  D = alpha * A * B + beta * C.
 //   prepare_kernel  : reference operands (1-bit values, reordered 2-bit-index metadata) -> prepared operand
 //   gemm_kernel     : main SMFMAC kernel (B staged through LDS, A expanded in registers)
-//   skinny_kernel   : split-K kernel for N <= 32 (decode shapes)
+//   skinny_kernel   : split-K kernel for N <= 64 (decode shapes)
 // Replaces the CUTLASS specialisations of the reference (csrc/kernel.h:13-72, csrc/threadblock.h:62-233,
 // csrc/warp.h:18-690) with code written for 64-wide wavefronts; nothing is translated from them.
 #include "onebit_device.h"
@@ -712,7 +712,7 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
 }
 
 // =====================================================================================================
-// skinny_kernel: N <= 32 (decode shapes). HBM-bound: every byte of the prepared operand is read once.
+// skinny_kernel: N <= 64 (decode shapes). HBM-bound: every byte of the prepared operand is read once.
 // Workgroup = NW wavefronts that share R row blocks (32 rows each) and split K among themselves: wavefront w
 // takes the K chunks (of 256) w, w + NW, w + 2 NW, ... Each wavefront stages B rows in a private 8 KiB LDS region
 // as a zero-padded fp16 image of NC columns (NC = 16: the 256 rows of a chunk; NC = 32: 128 rows, two images per
@@ -762,12 +762,13 @@ __device__ __forceinline__ u32x4_t skinny_load_piece(const _Float16* __restrict_
 template <int NW, int R, int MODE, int NC>
 __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(SkinnyArgs p) {
   constexpr int NT = 64 * NW;
-  constexpr int IMG_ROWS = kSkinnyRegion / (NC * 2);   // B rows per image: 256 or 128
-  constexpr int SUB = kChunkK / IMG_ROWS;              // images per chunk: 1 or 2
-  constexpr int IMG_STEPS = kStepsPerChunk / SUB;      // 32-wide K steps per image: 8 or 4
+  constexpr int IMG_ROWS = kSkinnyRegion / (NC * 2);   // B rows per image: 256, 128 or 64
+  constexpr int SUB = kChunkK / IMG_ROWS;              // images per chunk: 1, 2 or 4
+  constexpr int IMG_STEPS = kStepsPerChunk / SUB;      // 32-wide K steps per image: 8, 4 or 2
   constexpr int ROW_BYTES = NC * 2;
+  constexpr int NF = NC <= 32 ? 1 : NC / 32;           // 32-column fragments per image row
   constexpr int TILE_BYTES = kRowBlock * NC * 4;       // one fp32 partial tile
-  static_assert(NC == 16 || NC == 32, "image width");
+  static_assert(NC == 16 || NC == 32 || NC == 64, "image width");
   static_assert(MODE != kSkinnyB4 || NC == 16, "the 8-byte-row mode is for 16 columns");
   static_assert(R * TILE_BYTES <= kSkinnyRegion, "partial tiles reuse the wavefront's image memory");
   __shared__ __attribute__((aligned(16))) char bs[NW * kSkinnyRegion];
@@ -814,7 +815,7 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
       // columns n ... NC - 1 keep the zeros the image was cleared to
       const int valid = rows_valid_of(k_base) * n_cols, total = IMG_ROWS * n_cols;
       const _Float16* src = b_ptr + (size_t)k_base * n_cols;
-      constexpr int BATCH = NC == 32 ? 16 : 4;  // loads in flight per lane
+      constexpr int BATCH = NC >= 32 ? 16 : 4;  // loads in flight per lane
       int offset = elem_offset0;  // byte offset in the image of element e = lane + 64 i, kept without divisions
       int col = elem_col0;
       for (int e0 = lane; e0 < total; e0 += 64 * BATCH) {
@@ -844,23 +845,25 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
     for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4_t*>(region + (lane + i * 64) * 16) = v[i];
   };
 
-  float16_t acc[R];
+  float16_t acc[R][NF];
 #pragma unroll
   for (int r = 0; r < R; ++r)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[r][v] = 0.f;
+    for (int f = 0; f < NF; ++f)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[r][f][v] = 0.f;
   const uint32_t one = packed_one_in_vgpr();
   const int i16 = lane & 15, gb = lane >> 5;
   // NC == 16: lanes 16-31 and 48-63 would hold columns 16-31: they re-read columns 0-15 and are never stored
-  const int chunk8 = (NC == 32 ? ((lane & 31) >> 4) * 4 : 0) + (i16 & 3);  // 8-byte piece of the image row
+  const int chunk8 = (NC >= 32 ? ((lane & 31) >> 4) * 4 : 0) + (i16 & 3);  // 8-byte piece of the 32-column fragment
   const char* lane_ptr = region + (8 * gb + (i16 >> 2)) * ROW_BYTES + chunk8 * 8;
 
-  auto frag = [&](int image_step) __attribute__((always_inline)) {
+  auto frag = [&](int image_step, int f) __attribute__((always_inline)) {
     u32x8_t raw;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int row_const = image_step * 32 + 4 * (q & 1) + 16 * (q >> 1);
-      const u32x2_t t = lds_read_tr16(lane_ptr + row_const * ROW_BYTES);
+      const u32x2_t t = lds_read_tr16(lane_ptr + row_const * ROW_BYTES + f * 64);
       raw[2 * q] = t.x;
       raw[2 * q + 1] = t.y;
     }
@@ -871,17 +874,20 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
     constexpr int FIRST_STEP = decltype(sub_tag)::value * IMG_STEPS;
     // FG fragments (4 FG transpose reads) in flight, then their SMFMACs back to back; the scheduling barriers keep
     // the next group's reads from being hoisted (8 registers per fragment)
-    constexpr int FG = R >= 4 ? 2 : 4;
-    half16_t bfrag[FG];
+    constexpr int FG = (R >= 4 || NF > 1) ? 2 : 4;
+    half16_t bfrag[FG][NF];
     auto step = [&](auto step_tag) __attribute__((always_inline)) {
       constexpr int STEP = decltype(step_tag)::value;
 #pragma unroll
-      for (int r = 0; r < R; ++r)
+      for (int r = 0; r < R; ++r) {
 #if ONEBIT_EXP_SKINNY == 3
-        acc[r] = smfmac_step<STEP, false>(a[r], expand_signs<0>(a[0], one), bfrag[STEP % FG], acc[r]);
+        const half8_t av = expand_signs<0>(a[0], one);
 #else
-        acc[r] = smfmac_step<STEP, false>(a[r], expand_signs<STEP>(a[r], one), bfrag[STEP % FG], acc[r]);
+        const half8_t av = expand_signs<STEP>(a[r], one);
 #endif
+#pragma unroll
+        for (int f = 0; f < NF; ++f) acc[r][f] = smfmac_step<STEP, false>(a[r], av, bfrag[STEP % FG][f], acc[r][f]);
+      }
     };
     auto group = [&](auto first_tag) __attribute__((always_inline)) {
       constexpr int FIRST = decltype(first_tag)::value;  // step within the chunk
@@ -889,7 +895,9 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
       if (FIRST == 0)
 #endif
 #pragma unroll
-      for (int st = 0; st < FG; ++st) bfrag[st] = frag(FIRST - FIRST_STEP + st);
+      for (int st = 0; st < FG; ++st)
+#pragma unroll
+        for (int f = 0; f < NF; ++f) bfrag[st][f] = frag(FIRST - FIRST_STEP + st, f);
       step(std::integral_constant<int, FIRST>{});
       step(std::integral_constant<int, FIRST + 1>{});
       if constexpr (FG == 4) {
@@ -919,23 +927,31 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
     if (!kPrefetchB) load_b(k_base, breg);
     store_b(k_base, breg);  // after the previous image's fragment reads: LDS operations of a wavefront execute in order
 #if ONEBIT_EXP_SKINNY != 1
-    if (kPrefetchB) load_b(SUB == 2 ? k_base + IMG_ROWS : k_base + NW * kChunkK, breg);
+    if (kPrefetchB) load_b(SUB > 1 ? k_base + IMG_ROWS : k_base + NW * kChunkK, breg);
 #endif
     load_a(kc + NW, a_next);
 #if ONEBIT_EXP_SKINNY == 4
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r][0] += __builtin_bit_cast(float, a_cur[r].meta.x ^ a_cur[r].sign.y);
+    for (int r = 0; r < R; ++r) acc[r][0][0] += __builtin_bit_cast(float, a_cur[r].meta.x ^ a_cur[r].sign.y);
 #else
     compute(a_cur, std::integral_constant<int, 0>{});
-    if constexpr (SUB == 2) {
-      if (!kPrefetchB) {
-        __builtin_amdgcn_sched_barrier(0);  // the second image's loads stay behind the first image's SMFMACs
-        load_b(k_base + IMG_ROWS, breg);
+    // the chunk's further images (SUB - 1 of them)
+    auto further = [&](auto sub_tag) __attribute__((always_inline)) {
+      constexpr int S = decltype(sub_tag)::value;
+      if constexpr (S < SUB) {
+        const int image_base = k_base + S * IMG_ROWS;
+        if (!kPrefetchB) {
+          __builtin_amdgcn_sched_barrier(0);  // this image's loads stay behind the previous image's SMFMACs
+          load_b(image_base, breg);
+        }
+        store_b(image_base, breg);
+        if (kPrefetchB) load_b(S + 1 < SUB ? image_base + IMG_ROWS : k_base + NW * kChunkK, breg);
+        compute(a_cur, sub_tag);
       }
-      store_b(k_base + IMG_ROWS, breg);
-      if (kPrefetchB) load_b(k_base + NW * kChunkK, breg);
-      compute(a_cur, std::integral_constant<int, 1>{});
-    }
+    };
+    further(std::integral_constant<int, 1>{});
+    further(std::integral_constant<int, 2>{});
+    further(std::integral_constant<int, 3>{});
 #endif
 #pragma unroll
     for (int r = 0; r < R; ++r) a_cur[r] = a_next[r];
@@ -950,10 +966,12 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
 #pragma unroll
       for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int row = 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-          tile[(r * 32 + row) * NC + col] = acc[r][v];
-        }
+        for (int f = 0; f < NF; ++f)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int row = 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+            tile[(r * 32 + row) * NC + f * 32 + col] = acc[r][f][v];
+          }
     }
   }
   __syncthreads();
@@ -1125,6 +1143,11 @@ static hipError_t launch_skinny_mode(const SkinnyArgs& args, hipStream_t stream)
 template <int NW, int R>
 static hipError_t launch_skinny_cfg(const SkinnyArgs& args, hipStream_t stream) {
   const uintptr_t address = reinterpret_cast<uintptr_t>(args.b);
+  if (args.n > 32) {  // 64-column images; one partial tile fills the image memory
+    if (args.n == 64 && (address & 15) == 0) return launch_skinny_mode<NW, 1, kSkinnyBFull, 64>(args, stream);
+    if (args.n % 8 == 0 && (address & 15) == 0) return launch_skinny_mode<NW, 1, kSkinnyB8, 64>(args, stream);
+    return launch_skinny_mode<NW, 1, kSkinnyBScalar, 64>(args, stream);
+  }
   if (args.n > 16) {  // 32-column images; their two partial tiles per row block fill the image memory at R = 2
     constexpr int R32 = R > 2 ? 2 : R;
     if (args.n == 32 && (address & 15) == 0) return launch_skinny_mode<NW, R32, kSkinnyBFull, 32>(args, stream);

@@ -42,8 +42,9 @@ hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream);
 // dense fp16 (m x k) -> one-bit values `a` and metadata `e`; prune != 0 applies the 2:4 magnitude mask first
 hipError_t launch_pack(const void* w, void* a, void* e, int m, int k, int prune, int layout, hipStream_t stream);
 
-// Split-K kernel for n <= 32; rows_per_group (32, 64 or 128) = weight rows one workgroup covers (n > 16: 128 -> 64).
-constexpr int kSkinnyMaxN = 32;
+// Split-K kernel for n <= 64; rows_per_group (32, 64 or 128) = weight rows one workgroup covers (16 < n <= 32: at
+// most 64; n > 32: always 32).
+constexpr int kSkinnyMaxN = 64;
 hipError_t launch_skinny(SkinnyArgs args, int rows_per_group, hipStream_t stream);
 
 }  // namespace onebit

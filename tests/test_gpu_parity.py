@@ -194,11 +194,12 @@ def test_config3_decode(m, k, n):
 @pytest.mark.parametrize("rows", [32, 64, 128])
 @pytest.mark.parametrize("m,n,k", [(64, 1, 32), (192, 5, 800), (320, 8, 4128), (4096, 16, 4096), (1088, 4, 2048),
                                    (2240, 16, 8224), (128, 13, 12320), (192, 32, 800), (4096, 32, 4096),
-                                   (320, 17, 4128), (1088, 31, 2208), (64, 24, 32)])
+                                   (320, 17, 4128), (1088, 31, 2208), (64, 24, 32), (192, 64, 800),
+                                   (4096, 64, 4096), (320, 40, 4128), (1088, 63, 2208), (64, 33, 32)])
 def test_split_k_workgroup_shapes(rows, m, n, k):
     """every row-group size of the split-K kernel: chunk counts that do not divide among the wavefronts, a row
-    group past the last row block, K tails, every B staging mode (n = 32, 16, 8, 4 vector copies; element
-    copies), 16- and 32-column images"""
+    group past the last row block, K tails, every B staging mode (whole rows, padded 16-byte pieces, 8-byte rows,
+    element copies), 16-, 32- and 64-column images"""
     _native.set_skinny_rows(rows)
     a, meta = synthetic.make_weight(m, k, seed=rows + m + k)
     dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
@@ -217,6 +218,7 @@ def test_k_split_over_workgroups(splits, m, n, k):
     """main kernel with K split over workgroups (partial sums + ordered reduction): forced split counts that do and
     do not divide the chunk count, K tails, ragged N (generic variant), beta != 0, fp16 and fp32 results"""
     _native.set_split_k(splits)
+    _native.set_skinny_enabled(False)  # n = 40 would otherwise take the split-K kernel for small n
     a, meta = synthetic.make_weight(m, k, seed=splits + m + k)
     dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
     bi = synthetic.make_b(k, n, seed=n, kind="int")
@@ -327,7 +329,7 @@ def test_every_tile_configuration(tile, m, n, k):
     assert np.array_equal(got, exact)
 
 
-@pytest.mark.parametrize("n", [64, 32, 16, 8])  # main kernel's element-copy variant; split-K kernel's element mode
+@pytest.mark.parametrize("n", [72, 64, 32, 16, 8])  # main kernel's element-copy variant; split-K kernel's element mode
 def test_unaligned_b_pointer(n):
     m, k = 256, 128
     a, meta = synthetic.make_weight(m, k, seed=9)
