@@ -214,6 +214,8 @@ def main():
             note="no LDS or global memory in the loop; the gap to the nominal peak is clock throttling under load")
     if not args.no_decode:
         line["decode_n16"] = run_decode_rotating(11008, 4096, 16)
+        # the same kernel family where the weight is large enough for bandwidth, not latency, to set the time
+        line["decode_n16_large"] = run_decode_rotating(28672, 8192, 16, launches=500)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w, operands)
     print(json.dumps(line))
