@@ -138,6 +138,21 @@ __device__ __forceinline__ void lds_dma16_base(const void* base, uint32_t lane_o
                : "memory");
 }
 
+// Raw buffer loads: address = descriptor base (wave-uniform) + vector offset + scalar offset, so a loop that walks
+// memory needs scalar additions only and one vector register of lane offsets. The descriptor covers `bytes` bytes
+// (untyped 32-bit data format); the scalar offset takes no part in its range check, so callers keep every access
+// inside [base, base + bytes) themselves.
+typedef __amdgpu_buffer_rsrc_t buffer_t;
+__device__ __forceinline__ buffer_t make_buffer(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ u32x4_t buffer_load16(buffer_t buffer, uint32_t lane_offset, uint32_t uniform_offset) {
+  return __builtin_amdgcn_raw_buffer_load_b128(buffer, lane_offset, uniform_offset, 0);
+}
+__device__ __forceinline__ u32x2_t buffer_load8(buffer_t buffer, uint32_t lane_offset, uint32_t uniform_offset) {
+  return __builtin_amdgcn_raw_buffer_load_b64(buffer, lane_offset, uniform_offset, 0);
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter on gfx9");

@@ -782,15 +782,29 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   const uint8_t* __restrict__ prep = p.prep;
   const int n_cols = p.n, k_rows = p.k, kc_total = p.kc_total;
 
+  // The streaming loads go through buffer descriptors: wave-uniform base and offset in scalar registers, lane
+  // offsets in one vector register, no vector address arithmetic inside the K loop. One descriptor per row block
+  // (its kc_total blocks are consecutive, under 4 GiB for any K the argument checks admit) and one for B.
+  const uint32_t meta_off = (uint32_t)lane * 16u, sign_off = (uint32_t)kSignOffset + (uint32_t)lane * 8u;
+  buffer_t a_buffer[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    int rb = rb_first + r;
+    if (rb >= rb_total) rb = rb_total - 1;  // never stored
+    a_buffer[r] = make_buffer(prep + (size_t)rb * kc_total * kBlockBytes, (uint32_t)kc_total * kBlockBytes);
+  }
   auto load_a = [&](int kc, AChunk (&a)[R]) __attribute__((always_inline)) {
     if (kc >= kc_total) kc = kc_total - 1;  // never multiplied
+    const uint32_t block = (uint32_t)kc * kBlockBytes;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      int rb = rb_first + r;
-      if (rb >= rb_total) rb = rb_total - 1;  // never stored
-      a[r] = load_a_chunk(prep + ((size_t)rb * kc_total + kc) * kBlockBytes, lane);
+      a[r].meta = buffer_load16(a_buffer[r], meta_off, block);
+      a[r].sign = buffer_load8(a_buffer[r], sign_off, block);
     }
   };
+  const size_t b_bytes = (size_t)k_rows * n_cols * 2;
+  const bool b_fits = b_bytes < (size_t(1) << 32);  // else every image takes the general path
+  const buffer_t b_buffer = make_buffer(b_ptr, b_fits ? (uint32_t)b_bytes : 0u);
   auto rows_valid_of = [&](int k_base) __attribute__((always_inline)) {
     const int rows = k_rows - k_base;
     return rows < 0 ? 0 : (rows > IMG_ROWS ? IMG_ROWS : rows);
@@ -805,6 +819,13 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   // multiplied; element mode: loaded and stored in one go when the image is due.
   auto load_b = [&](int k_base, u32x4_t (&v)[8]) __attribute__((always_inline)) {
     if (MODE == kSkinnyBScalar) return;
+    if (MODE == kSkinnyBFull && b_fits && k_base + IMG_ROWS <= k_rows) {
+      // the whole image lies inside B (wave-uniform test): 8 KiB of consecutive memory, no per-piece checks
+      const uint32_t image = (uint32_t)k_base * (NC * 2);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = buffer_load16(b_buffer, meta_off + 1024u * i, image);
+      return;
+    }
     const int rows_valid = rows_valid_of(k_base);
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = skinny_load_piece<NC>(b_ptr, n_cols, MODE, k_base, rows_valid, lane + i * 64);
