@@ -205,9 +205,14 @@ def main():
                            f"{DENSE_F16_PEAK_TFLOPS:.1f}); the same fraction as executed FLOPs MNK against the dense peak",
                       hbm_gbps_algorithmic=algorithmic_bytes(m, n, k, w["beta"]) / kernel_s / 1e9),
         wall_ms_per_step=wall_s * 1e3)
+    from onebitsparsemul_amd import _native
+    cus, khz = _native.device_info()
+    line["device"] = dict(name=torch.cuda.get_device_name(0), compute_units=cus, clock_mhz=khz / 1e3,
+                          smfmac_peak_from_device_tflops=2 * cus * khz * 1e3 * 4096 / 1e12,
+                          note="peak = CUs x clock x 4096 dense fp16 FLOP/clk/CU x 2 (sparse); roofline.peak uses the "
+                               "published 256 CUs x 2.4 GHz")
     if not args.no_ceiling:
         # register-only SMFMAC loops: what the chip sustains under matrix load, which depends on the operand values
-        from onebitsparsemul_amd import _native
         line["smfmac_register_loop_tflops"] = dict(
             benchmark_distribution=max(_native.measure_smfmac_rate(True, 50000) for _ in range(4)),
             constant_operands=max(_native.measure_smfmac_rate(False, 50000) for _ in range(4)),

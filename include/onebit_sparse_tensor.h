@@ -105,6 +105,10 @@ void onebit_sparse_set_split_k(int splits);
  * this is the practical ceiling next to the nominal peak. Allocates and frees its own device buffers; synchronous. */
 int onebit_sparse_measure_smfmac_rate(int random_operands, int iterations, double *dense_equiv_tflops);
 
+/* Diagnostic, no counterpart in the reference: compute units and peak engine clock (kHz) of the current device, the
+ * two figures the SMFMAC peak is computed from (units x clock x 4096 dense fp16 FLOP per clock per unit x 2). */
+int onebit_sparse_device_info(int *compute_units, int *clock_khz);
+
 #ifdef __cplusplus
 }
 #endif

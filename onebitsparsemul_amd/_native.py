@@ -16,7 +16,7 @@ EXPORTS = (
     "onebit_sparse_matmul", "onebit_sparse_matmul_ex", "onebit_sparse_prepared_bytes", "onebit_sparse_prepare",
     "onebit_sparse_matmul_prepared", "onebit_sparse_pack", "onebit_sparse_last_error", "onebit_sparse_set_tile_config",
     "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_set_split_k",
-    "onebit_sparse_measure_smfmac_rate",
+    "onebit_sparse_measure_smfmac_rate", "onebit_sparse_device_info",
 )
 
 _lib = None
@@ -51,6 +51,8 @@ def lib():
         L.onebit_sparse_set_skinny_rows.argtypes = [i32]
         L.onebit_sparse_set_split_k.restype = None
         L.onebit_sparse_set_split_k.argtypes = [i32]
+        L.onebit_sparse_device_info.restype = i32
+        L.onebit_sparse_device_info.argtypes = [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
         L.onebit_sparse_measure_smfmac_rate.restype = i32
         L.onebit_sparse_measure_smfmac_rate.argtypes = [i32, i32, ctypes.POINTER(ctypes.c_double)]
         _lib = L
@@ -179,3 +181,10 @@ def pack_weight(weight, prune=True, layout=META_REFERENCE):
         _check(lib().onebit_sparse_pack(weight.data_ptr(), m, k, 1 if prune else 0, a.data_ptr(), meta.data_ptr(), layout,
                                         _stream(weight)))
     return a, meta
+
+
+def device_info():
+    """(compute units, peak engine clock in kHz) of the current device."""
+    cus, khz = ctypes.c_int(0), ctypes.c_int(0)
+    _check(lib().onebit_sparse_device_info(ctypes.byref(cus), ctypes.byref(khz)))
+    return cus.value, khz.value

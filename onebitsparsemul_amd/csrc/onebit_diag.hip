@@ -103,3 +103,12 @@ done:
   (void)hipFree(pidx);
   return rc;
 }
+
+extern "C" int onebit_sparse_device_info(int* compute_units, int* clock_khz) {
+  if (!compute_units || !clock_khz) return ONEBIT_ERR_ARGUMENT;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return ONEBIT_ERR_HIP;
+  if (hipDeviceGetAttribute(compute_units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return ONEBIT_ERR_HIP;
+  if (hipDeviceGetAttribute(clock_khz, hipDeviceAttributeClockRate, device) != hipSuccess) return ONEBIT_ERR_HIP;
+  return ONEBIT_OK;
+}

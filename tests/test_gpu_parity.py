@@ -155,6 +155,14 @@ def _sampled_rows_check(prep, dense, size, seed):
     rows.sort()
     ref = dense.numpy()[rows].astype(np.float64) @ b.cpu().numpy().astype(np.float64)
     _assert_close(d[torch.from_numpy(rows).cuda()].cpu().numpy(), ref)
+    # the whole output against a dense fp16 library GEMM of the decompressed weight on the GPU (another code path).
+    # Both results are fp32 sums rounded once to fp16: |d - lib| <= 1e-3 |lib| + 1e-3 sqrt(K/2) element by element
+    # (fp16 rounding alone is 4.9e-4 relative; sqrt(K/2) is the scale of one output element)
+    lib = torch.matmul(dense.cuda().to(torch.float16), b)
+    err = (d.float() - lib.float()).abs()
+    bound = 1e-3 * lib.float().abs() + 1e-3 * float(np.sqrt(k / 2))
+    assert bool((err <= bound).all()), f"{int((err > bound).sum())} elements off the library GEMM"
+    del lib, err, bound
     # linearity, exact: integer B1, B2
     b1 = synthetic.make_b(k, n, seed=seed + 1, kind="int", device="cuda")
     b2 = synthetic.make_b(k, n, seed=seed + 2, kind="int", device="cuda")
