@@ -89,8 +89,8 @@ int pick_tile(int m, int n) {
   const int forced = g_tile_config.load();
   if (forced >= 0) return forced;
   // Largest tile that still gives every CU its share of workgroups (measured on MI355X, interleaved runs):
-  // 512 x 128 with eight wavefronts (one workgroup per CU) from 256 tiles on - 8192^3: 2.09 PF, 4096^3: 1.79 PF
-  // against 1.66 PF for 256 x 128; 256 x 128 with four wavefronts (two workgroups per CU) from 512 tiles on;
+  // 512 x 128 with eight wavefronts (one workgroup per CU) from 256 tiles on - 8192^3: 2.2 PF, 4096^3: 2.03 PF
+  // against 1.91 PF for 256 x 128 (sustained clock); 256 x 128 with four wavefronts (two workgroups per CU) from 512 tiles on;
   // 128 x 128 (64 x 64 per wavefront) below that - 4096 x 2048 x 4096 is 12 % faster with it than with 256 x 128.
   auto tiles = [&](int bm, int bn) { return (long)((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
   if (tiles(512, 128) >= 256) return onebit::kTile512x128w8;
