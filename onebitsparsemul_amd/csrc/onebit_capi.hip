@@ -88,13 +88,16 @@ int check_dtype(int c_dtype, int d_dtype) {
 int pick_tile(int m, int n) {
   const int forced = g_tile_config.load();
   if (forced >= 0) return forced;
-  // Largest tile that still gives every CU its share of workgroups (measured on MI355X, interleaved runs):
+  // Largest tile that still gives every CU its share of workgroups (measured on MI355X at the sustained clock):
   // 512 x 128 with eight wavefronts (one workgroup per CU) from 256 tiles on - 8192^3: 2.2 PF, 4096^3: 2.03 PF
-  // against 1.91 PF for 256 x 128 (sustained clock); 256 x 128 with four wavefronts (two workgroups per CU) from 512 tiles on;
-  // 128 x 128 (64 x 64 per wavefront) below that - 4096 x 2048 x 4096 is 12 % faster with it than with 256 x 128.
+  // against 1.91 PF for 256 x 128 - unless its last round of 256 would be mostly empty (11008 x 2048 x 4096: 352
+  // tiles, 117 us against 102 us for 256 x 128); 256 x 128 with four wavefronts from 256 tiles on (8192 x 1024 x
+  // 8192: 76 us against 83 us for 128 x 128); 128 x 128 (64 x 64 per wavefront, two workgroups per CU) below that.
   auto tiles = [&](int bm, int bn) { return (long)((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
-  if (tiles(512, 128) >= 256) return onebit::kTile512x128w8;
-  if (tiles(256, 128) >= 512) return onebit::kTile256x128w;
+  const long big = tiles(512, 128);
+  // its rounds of 256 workgroups at least 77 % full (5120^3, 78 %: 140 us against 151; 6144^3, 75 %: 255 against 234)
+  if (big >= 256 && big * 100 >= ((big + 255) / 256) * 256 * 77) return onebit::kTile512x128w8;
+  if (tiles(256, 128) >= 256) return onebit::kTile256x128w;
   return onebit::kTile128x128s;
 }
 
