@@ -97,7 +97,13 @@ int pick_tile(int m, int n) {
   const long big = tiles(512, 128);
   // its rounds of 256 workgroups at least 77 % full (5120^3, 78 %: 140 us against 151; 6144^3, 75 %: 255 against 234)
   if (big >= 256 && big * 100 >= ((big + 255) / 256) * 256 * 77) return onebit::kTile512x128w8;
-  if (tiles(256, 128) >= 256) return onebit::kTile256x128w;
+  // With at most one workgroup per CU the eight-wavefront forms of the small tiles run two wavefronts per SIMD
+  // instead of one: 256 x 128 (4096 x 2048 x 4096: 42.4 us against 46.3), 128 x 128 (2048^3: 14.9 against 15.6,
+  // 1024^3: 8.4 against 9.2, 512^3: 5.9 against 6.6).
+  const long mid = tiles(256, 128);
+  if (mid >= 512) return onebit::kTile256x128w;
+  if (mid >= 256) return onebit::kTile256x128w8;
+  if (tiles(128, 128) <= 256) return onebit::kTile128x128w8;
   return onebit::kTile128x128s;
 }
 
@@ -110,7 +116,7 @@ int pick_splits(int m, int n, int k, int tile) {
   const int chunks = (k + onebit::kChunkK - 1) / onebit::kChunkK;
   const int forced = g_split_k.load();
   if (forced >= 1) return forced < chunks ? forced : chunks;
-  if (tile != onebit::kTile128x128s) return 1;
+  if (tile != onebit::kTile128x128s && tile != onebit::kTile128x128w8) return 1;
   const double tiles = (double)((m + 127) / 128) * ((n + 127) / 128);
   const double result_bytes = 4.0 * m * n;
   int best = 1;
