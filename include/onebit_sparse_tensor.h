@@ -98,6 +98,11 @@ void onebit_sparse_set_skinny_rows(int rows);
  * device and stream (grown with hipMalloc on first use: warm up before capturing the call in a HIP graph) and adds
  * them in split order, so results do not depend on timing. */
 void onebit_sparse_set_split_k(int splits);
+/* B whose rows are not 16-byte aligned (n % 8 != 0 or an unaligned base) and n beyond the split-K kernel's range:
+ * 1 (default) = the main kernel reads a copy of B with rows padded to a multiple of 8 columns, made by one extra
+ * pass into a library-owned buffer kept per device and stream (same rules as the K-split buffer); 0 = the main
+ * kernel's element-copy variant reads B in place (much slower; always used when k * n < 65536). */
+void onebit_sparse_set_pad_b(int enabled);
 
 /* Diagnostic, no counterpart in the reference: sustained rate of v_smfmac_f32_32x32x32_f16 in a register-only
  * loop on the current device (one wavefront per SIMD, `iterations` x 16 instructions each), in dense-equivalent

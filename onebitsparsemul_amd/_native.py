@@ -15,7 +15,7 @@ META_REFERENCE, META_CUTLASS, META_LOGICAL = 0, 1, 2
 EXPORTS = (
     "onebit_sparse_matmul", "onebit_sparse_matmul_ex", "onebit_sparse_prepared_bytes", "onebit_sparse_prepare",
     "onebit_sparse_matmul_prepared", "onebit_sparse_pack", "onebit_sparse_last_error", "onebit_sparse_set_tile_config",
-    "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_set_split_k",
+    "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_set_split_k", "onebit_sparse_set_pad_b",
     "onebit_sparse_measure_smfmac_rate", "onebit_sparse_device_info",
 )
 
@@ -51,6 +51,8 @@ def lib():
         L.onebit_sparse_set_skinny_rows.argtypes = [i32]
         L.onebit_sparse_set_split_k.restype = None
         L.onebit_sparse_set_split_k.argtypes = [i32]
+        L.onebit_sparse_set_pad_b.restype = None
+        L.onebit_sparse_set_pad_b.argtypes = [i32]
         L.onebit_sparse_device_info.restype = i32
         L.onebit_sparse_device_info.argtypes = [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
         L.onebit_sparse_measure_smfmac_rate.restype = i32
@@ -158,6 +160,10 @@ def set_skinny_rows(rows):
 
 def set_split_k(splits):
     lib().onebit_sparse_set_split_k(splits)
+
+
+def set_pad_b(enabled):
+    lib().onebit_sparse_set_pad_b(1 if enabled else 0)
 
 
 def measure_smfmac_rate(random_operands=True, iterations=50000):

@@ -20,6 +20,7 @@ std::atomic<int> g_tile_config{-1};
 std::atomic<int> g_skinny_enabled{1};
 std::atomic<int> g_skinny_rows{-1};
 std::atomic<int> g_split_k{-1};
+std::atomic<int> g_pad_b{1};
 
 int fail(int code, const char* fmt, ...) {
   char buf[512];
@@ -53,6 +54,8 @@ struct DeviceState {
   // fp32 partial sums of the K-split passes: one buffer per stream, so that calls on different streams do not
   // share one (calls on the same stream are ordered)
   std::map<hipStream_t, Buffer> split_ws;
+  // B with rows padded to a multiple of 8 columns (operands the asynchronous copies cannot read in place), per stream
+  std::map<hipStream_t, Buffer> b_pad;
 };
 DeviceState g_dev[kMaxDevices];
 
@@ -175,18 +178,30 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
   args.d_f16 = d_dtype == ONEBIT_DTYPE_F16;
   const int tile = pick_tile(m, n);
   const int splits = pick_splits(m, n, k, tile);
-  if (splits > 1) {
-    const int cps = (kc_total + splits - 1) / splits;
-    args.chunks_per_split = cps;
-    args.splits = (kc_total + cps - 1) / cps;  // every split non-empty
+  // B rows that are not 16-byte aligned: pad a copy (one extra pass over B) unless the problem is too small for that
+  // to pay against the element-copy variant of the kernel
+  const bool b_in_place = n % 8 == 0 && (reinterpret_cast<uintptr_t>(b) & 15) == 0;
+  const bool pad_b = !b_in_place && (size_t)k * n >= 65536 && g_pad_b.load();
+  if (splits > 1 || pad_b) {
     int device = 0;
     ONEBIT_HIP(hipGetDevice(&device));
     if (device < 0 || device >= kMaxDevices) return fail(ONEBIT_ERR_ARGUMENT, "device ordinal %d not supported", device);
     DeviceState& st = g_dev[device];
     std::lock_guard<std::mutex> lock(st.mu);
-    Buffer& ws = st.split_ws[stream];
-    if (int rc = grow(&ws.ptr, &ws.bytes, (size_t)args.splits * m * n * sizeof(float)); rc != ONEBIT_OK) return rc;
-    args.split_ws = static_cast<float*>(ws.ptr);
+    if (splits > 1) {
+      const int cps = (kc_total + splits - 1) / splits;
+      args.chunks_per_split = cps;
+      args.splits = (kc_total + cps - 1) / cps;  // every split non-empty
+      Buffer& ws = st.split_ws[stream];
+      if (int rc = grow(&ws.ptr, &ws.bytes, (size_t)args.splits * m * n * sizeof(float)); rc != ONEBIT_OK) return rc;
+      args.split_ws = static_cast<float*>(ws.ptr);
+    }
+    if (pad_b) {
+      Buffer& pb = st.b_pad[stream];
+      const size_t ldb = (size_t)(n + 7) / 8 * 8;
+      if (int rc = grow(&pb.ptr, &pb.bytes, (size_t)k * ldb * sizeof(_Float16)); rc != ONEBIT_OK) return rc;
+      args.b_pad = static_cast<_Float16*>(pb.ptr);
+    }
     ONEBIT_HIP(onebit::launch_gemm(args, tile, stream));
     return ONEBIT_OK;
   }
@@ -204,6 +219,7 @@ void onebit_sparse_set_tile_config(int tile_config) { g_tile_config.store(tile_c
 void onebit_sparse_set_skinny_enabled(int enabled) { g_skinny_enabled.store(enabled ? 1 : 0); }
 void onebit_sparse_set_skinny_rows(int rows) { g_skinny_rows.store(rows); }
 void onebit_sparse_set_split_k(int splits) { g_split_k.store(splits); }
+void onebit_sparse_set_pad_b(int enabled) { g_pad_b.store(enabled ? 1 : 0); }
 
 size_t onebit_sparse_prepared_bytes(int m, int k) {
   if (m <= 0 || k <= 0) return 0;

@@ -439,12 +439,12 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
       const int row = slot / CH, pc = slot % CH;
       const int lc = pc ^ chunk_swizzle<BN>(row);
       int col = 8 * lc;
-      if (n0 + col >= p.n) col = 0;  // columns past N: any valid address will do, the results are not stored
-      b_off[i] = (uint32_t)(row * p.n + col) * 2u;
+      if (n0 + col >= p.ldb) col = 0;  // columns past the row: any valid address will do, the results are not stored
+      b_off[i] = (uint32_t)(row * p.ldb + col) * 2u;
       copy_row[i] = row;
       lds_dst[i] = smem_base + (NW * i + wave) * 1024;
     }
-    const size_t stage_stride = (size_t)kStageK * p.n * 2;
+    const size_t stage_stride = (size_t)kStageK * p.ldb * 2;
     const char* b_stage = reinterpret_cast<const char*>(p.b) + (size_t)n0 * 2 +
                           (size_t)chunk_begin * kStages * stage_stride;  // advances one stage per copy
     const char* zeros = reinterpret_cast<const char*>(g_zero16);
@@ -1016,6 +1016,24 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
 }
 
 // =====================================================================================================
+// pad_b_kernel: copies B (k x n, row stride n, any alignment) into rows of ldb = round_up(n, 8) halves, zeros in the
+// padding columns, so that every row starts 16-byte aligned for the asynchronous copies of the main kernel.
+// One thread per 16-byte piece of the destination.
+// =====================================================================================================
+__global__ __launch_bounds__(256) void pad_b_kernel(const _Float16* __restrict__ b, _Float16* __restrict__ dst, int k,
+                                                    int n, int ldb) {
+  const int pieces_per_row = ldb / 8;
+  const size_t piece = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (piece >= (size_t)k * pieces_per_row) return;
+  const size_t row = piece / pieces_per_row;
+  const int col0 = (int)(piece % pieces_per_row) * 8;
+  half8_t v;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = col0 + j < n ? b[row * n + col0 + j] : (_Float16)0.f;
+  *reinterpret_cast<half8_t*>(dst + row * ldb + col0) = v;
+}
+
+// =====================================================================================================
 // splitk_reduce_kernel: d = alpha * (sum over splits, in split order, of the fp32 partial sums) + beta * c.
 // Elementwise over the m * n results; VEC = 4 when the element count and the alignment of c and d allow it.
 // =====================================================================================================
@@ -1102,9 +1120,9 @@ static hipError_t launch_gemm_cfg(GemmArgs args, hipStream_t stream) {
 }
 
 static hipError_t launch_gemm_pass(GemmArgs args, int tile_config, hipStream_t stream) {
-  const bool aligned = (args.n % 8 == 0) && ((reinterpret_cast<uintptr_t>(args.b) & 15) == 0);
+  const bool aligned = (args.ldb % 8 == 0) && ((reinterpret_cast<uintptr_t>(args.b) & 15) == 0);
   // the coalesced epilogue moves 16 bytes per lane: n % 8 == 0 keeps every row start aligned when the bases are
-  args.vector_epilogue = (reinterpret_cast<uintptr_t>(args.d) & 15) == 0 &&
+  args.vector_epilogue = args.n % 8 == 0 && (reinterpret_cast<uintptr_t>(args.d) & 15) == 0 &&
                          (args.beta == 0.f || (reinterpret_cast<uintptr_t>(args.c) & 15) == 0);
   if (!aligned) return launch_gemm_cfg<4, 1, 1, 4, false>(args, stream);
   switch (tile_config) {
@@ -1126,6 +1144,17 @@ static hipError_t launch_gemm_pass(GemmArgs args, int tile_config, hipStream_t s
 
 hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
   if (prepared_bytes(args.m, args.k) >= (size_t(1) << 32)) return hipErrorInvalidValue;  // 32-bit copy offsets
+  args.ldb = args.n;
+  const bool aligned = (args.n % 8 == 0) && ((reinterpret_cast<uintptr_t>(args.b) & 15) == 0);
+  if (!aligned && args.b_pad) {
+    const int ldb = (args.n + 7) / 8 * 8;
+    const size_t pieces = (size_t)args.k * (ldb / 8);
+    hipLaunchKernelGGL(pad_b_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, stream, args.b, args.b_pad,
+                       args.k, args.n, ldb);
+    if (hipError_t st = hipGetLastError(); st != hipSuccess) return st;
+    args.b = args.b_pad;
+    args.ldb = ldb;
+  }
   const int chunks = (args.k + kChunkK - 1) / kChunkK;
   if (args.splits <= 1) {
     args.splits = 1;

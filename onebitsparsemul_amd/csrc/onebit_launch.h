@@ -22,6 +22,12 @@ struct GemmArgs {
   int splits;
   int chunks_per_split;
   float* split_ws;
+  // B whose rows are not 16-byte aligned (n % 8 != 0, or a base address that is not) cannot feed the asynchronous
+  // 16-byte copies. If b_pad is set (at least k * round_up(n, 8) halves, 16-byte aligned), the launcher first copies
+  // B into it with rows padded to a multiple of 8 columns and the main kernel reads that; otherwise such operands
+  // take the slower element-copy variant. ldb (elements between B rows) is filled by the launcher.
+  _Float16* b_pad;
+  int ldb;
 };
 
 struct SkinnyArgs {

@@ -26,11 +26,13 @@ def _defaults():
     _native.set_skinny_enabled(True)
     _native.set_skinny_rows(-1)
     _native.set_split_k(-1)
+    _native.set_pad_b(True)
     yield
     _native.set_tile_config(-1)
     _native.set_skinny_enabled(True)
     _native.set_skinny_rows(-1)
     _native.set_split_k(-1)
+    _native.set_pad_b(True)
 
 
 def _gpu(*ts):
@@ -369,6 +371,32 @@ def test_unaligned_value_bits_pointer():
     _native.matmul_ex(ad, bi.cuda(), meta.cuda(), d, m, n, k)
     torch.cuda.synchronize()
     assert np.array_equal(d.cpu().numpy(), exact)
+
+
+@pytest.mark.parametrize("pad", [True, False])
+@pytest.mark.parametrize("m,n,k,offset", [(512, 1001, 1056, 0), (1024, 203, 4128, 0), (256, 264, 512, 1),
+                                          (384, 100, 2048, 3)])
+def test_b_rows_not_16_byte_aligned(pad, m, n, k, offset):
+    """n % 8 != 0 or an unaligned B base, beyond the split-K kernel's n: the padded copy of B feeding the main
+    kernel (with and without a K split) and the element-copy variant give the oracle's result, with beta != 0"""
+    _native.set_pad_b(pad)
+    a, meta = synthetic.make_weight(m, k, seed=m + n + k)
+    dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
+    bi = synthetic.make_b(k, n, seed=n, kind="int")
+    ci = synthetic.make_c(m, n, seed=n + 1, dtype=torch.float32).round()
+    exact = oracle.host_gemm(dense, bi.numpy(), c=ci.numpy(), alpha=-1.0, beta=1.0, d_dtype=oracle.F32, acc="f32")
+    ad, md = _gpu(a, meta)
+    prep = _native.prepare(ad, md, m, k)
+    storage = torch.zeros(k * n + 16, dtype=torch.float16, device="cuda")
+    bd = storage[offset:offset + k * n].view(k, n)
+    bd.copy_(bi.cuda())
+    for out_dtype in (torch.float32, torch.float16):
+        d = torch.full((m, n), float("nan"), dtype=out_dtype, device="cuda")
+        _native.matmul_prepared(prep, bd, d, m, n, k, c=ci.cuda(), alpha=-1.0, beta=1.0)
+        torch.cuda.synchronize()
+        want = exact if out_dtype == torch.float32 else exact.astype(np.float16)
+        assert np.array_equal(d.cpu().numpy(), want)
+    assert torch.equal(bd.cpu(), bi)  # B itself is untouched
 
 
 def test_reference_benchmark_dataset():
