@@ -215,7 +215,8 @@ int ob_sparse_to_dense(const float *sparse, const int16_t *meta_reordered, int m
  * _semi_structured_conversions.py:286-314. The reference prunes the first two entries of an ascending
  * argsort whose order among equal keys is unspecified; this restatement uses the stable order (lower
  * index pruned first), which reproduces the only tie case the reference documents (all-ones weights ->
- * mask 0,0,1,1: tests/python/test_sparse.py:23-24). */
+ * mask 0,0,1,1: tests/python/test_sparse.py:23-24) and is what PyTorch's CPU argsort returns for all 256 rank
+ * patterns of four magnitudes (tests/test_oracle_format.py checks that against PyTorch's own routine). */
 void ob_mask_creator(const float *w, int64_t numel, float *mask) {
   for (int64_t g = 0; g < numel / 4; g++) {
     int order[4] = {0, 1, 2, 3};

@@ -64,6 +64,24 @@ def test_kat_compress_rows(oracle_lib, kat):
     assert np.array_equal(oracle_lib.sparse_to_dense(sparse, meta), dense)
 
 
+def test_mask_tie_rule_is_what_the_reference_expression_gives_on_this_torch(oracle_lib):
+    """The reference prunes `torch.argsort(|w|, dim=1)[:, :2]` of every group of four (unstable sort,
+    _semi_structured_conversions.py:308-309). On the CPU build of PyTorch in this image that call returns the
+    stable order for every one of the 256 rank patterns of four magnitudes (checked here with PyTorch's own
+    routine, for the dtypes a weight can have and for small and large row counts), so the oracle's rule - among
+    equal magnitudes the lower index is pruned first - is the reference's result in this environment."""
+    import itertools
+    import torch
+    patterns = torch.tensor(list(itertools.product(range(4), repeat=4)), dtype=torch.float32)
+    for repeats in (1, 300):
+        x = patterns.repeat(repeats, 1)
+        for dtype in (torch.float32, torch.float16, torch.bfloat16):
+            unstable = torch.argsort(x.to(dtype), dim=1)[:, :2]
+            mask = torch.ones_like(x).scatter_(1, unstable, 0.0)
+            got = oracle_lib.mask_creator(x.numpy())
+            assert np.array_equal(got, mask.numpy())
+
+
 def test_kat_mask(oracle_lib, kat):
     for row, mask in zip(kat["dense_rows"], kat["mask_rows"]):
         got = oracle_lib.mask_creator(np.array([row], dtype=np.float32))
