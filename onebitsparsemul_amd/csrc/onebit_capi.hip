@@ -110,29 +110,50 @@ int pick_tile(int m, int n) {
   return onebit::kTile128x128s;
 }
 
-// Number of K splits for the main kernel. Few tiles and a long K leave most compute units idle and make the
-// time the length of one workgroup's K loop; splitting K fills the GPU at the price of a second launch and of
-// writing and re-reading fp32 partial sums. Chosen with a cost model fitted to measurements of the 128 x 128
-// tile on MI355X (microseconds): 1.4 per 256-wide chunk of one workgroup's K loop, times the rounds of 512
-// resident workgroups; a split adds 5 for the second launch and the partial sums move at about 1.5 TB/s.
-int pick_splits(int m, int n, int k, int tile) {
+// Tile and number of K splits of the main kernel. Few tiles and a long K leave most compute units idle and make
+// the time the length of one workgroup's K loop; a smaller tile (64 x 128) or a split of K fills the GPU, the split
+// at the price of a second launch and of writing and re-reading fp32 partial sums. In that regime (fewer than 256
+// tiles of 256 x 128) the choice comes from a cost model fitted to measurements on MI355X, in microseconds: one
+// workgroup's K loop takes 1.4 per 256-wide chunk with the 128 x 128 tile and 0.95 with the 64 x 128 tile, times
+// the rounds of one workgroup per CU; a split adds 5 for the second launch and the partial sums move at about 3 TB/s.
+struct GemmPlan {
+  int tile;
+  int splits;
+};
+
+GemmPlan plan_gemm(int m, int n, int k) {
   const int chunks = (k + onebit::kChunkK - 1) / onebit::kChunkK;
-  const int forced = g_split_k.load();
-  if (forced >= 1) return forced < chunks ? forced : chunks;
-  if (tile != onebit::kTile128x128s && tile != onebit::kTile128x128w8) return 1;
-  const double tiles = (double)((m + 127) / 128) * ((n + 127) / 128);
+  const int forced_tile = g_tile_config.load();
+  const int forced_splits = g_split_k.load();
+  const int tile = pick_tile(m, n);
+  auto small_tile = [](int t) {
+    return t == onebit::kTile128x128s || t == onebit::kTile128x128w8 || t == onebit::kTile64x128;
+  };
+  if (!small_tile(tile) || forced_splits >= 1) {
+    int splits = forced_splits >= 1 ? forced_splits : 1;
+    if (splits > chunks) splits = chunks;
+    return GemmPlan{tile, splits};
+  }
   const double result_bytes = 4.0 * m * n;
-  int best = 1;
+  GemmPlan best{tile, 1};
   double best_us = 1e30;
-  for (int s : {1, 2, 3, 4, 6, 8, 12, 16}) {
-    if (s > chunks) break;
-    const int per_split = (chunks + s - 1) / s;
-    const double rounds = (double)(long)((tiles * s + 511) / 512);
-    double us = 1.4 * per_split * rounds;
-    if (s > 1) us += 5.0 + (s + 1) * result_bytes / 1.5e6;
-    if (us < best_us) {
-      best_us = us;
-      best = s;
+  const int candidates[2] = {tile, forced_tile >= 0 ? tile : (int)onebit::kTile64x128};
+  for (int c = 0; c < 2; ++c) {
+    const int t = candidates[c];
+    if (c == 1 && t == candidates[0]) break;
+    const bool low = t == onebit::kTile64x128;
+    const double chunk_us = low ? 0.95 : 1.4;
+    const double tiles = (double)((m + (low ? 63 : 127)) / (low ? 64 : 128)) * ((n + 127) / 128);
+    for (int s : {1, 2, 3, 4, 6, 8, 12, 16}) {
+      if (s > chunks) break;
+      const int per_split = (chunks + s - 1) / s;
+      const double rounds = (double)(long)((tiles * s + 255) / 256);
+      double us = chunk_us * per_split * rounds;
+      if (s > 1) us += 5.0 + (s + 1) * result_bytes / 3.0e6;
+      if (us < best_us) {
+        best_us = us;
+        best = GemmPlan{t, s};
+      }
     }
   }
   return best;
@@ -176,8 +197,9 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
   args.alpha = alpha; args.beta = beta;
   args.c_f16 = c_dtype == ONEBIT_DTYPE_F16;
   args.d_f16 = d_dtype == ONEBIT_DTYPE_F16;
-  const int tile = pick_tile(m, n);
-  const int splits = pick_splits(m, n, k, tile);
+  const GemmPlan plan = plan_gemm(m, n, k);
+  const int tile = plan.tile;
+  const int splits = plan.splits;
   // B rows that are not 16-byte aligned: pad a copy (one extra pass over B) unless the problem is too small for that
   // to pay against the element-copy variant of the kernel
   const bool b_in_place = n % 8 == 0 && (reinterpret_cast<uintptr_t>(b) & 15) == 0;

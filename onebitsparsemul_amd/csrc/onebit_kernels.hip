@@ -1138,6 +1138,7 @@ static hipError_t launch_gemm_pass(GemmArgs args, int tile_config, hipStream_t s
     case kTile512x128w8: return launch_gemm_cfg<4, 2, 4, 2, true>(args, stream);
     case kTile256x128w8: return launch_gemm_cfg<4, 2, 2, 2, true>(args, stream);
     case kTile128x128w8: return launch_gemm_cfg<2, 4, 2, 1, true>(args, stream);
+    case kTile64x128: return launch_gemm_cfg<2, 2, 1, 2, true>(args, stream);
     default: return hipErrorInvalidValue;
   }
 }
