@@ -399,6 +399,37 @@ def test_b_rows_not_16_byte_aligned(pad, m, n, k, offset):
     assert torch.equal(bd.cpu(), bi)  # B itself is untouched
 
 
+@pytest.mark.parametrize("m,n,k", [(1024, 16, 2048), (512, 256, 512), (256, 128, 8192), (512, 1001, 1056), (2048, 64, 4096)])
+def test_hip_graph_replays_match_eager(m, n, k):
+    """a prepared call captured in a HIP graph (after one eager call, which sizes the library's K-split and padded-B
+    buffers): every replay, with new B values written between replays, equals the eager result; covers the
+    split-K kernel, the main kernel, its K split over workgroups and the padded copy of B"""
+    a, meta = synthetic.make_weight(m, k, seed=m + n)
+    ad, md = _gpu(a, meta)
+    prep = _native.prepare(ad, md, m, k)
+    b = torch.zeros((k, n), dtype=torch.float16, device="cuda")
+    d = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        _native.matmul_prepared(prep, b, d, m, n, k)  # eager warm-up on the capture stream
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            _native.matmul_prepared(prep, b, d, m, n, k)
+    for replay in range(4):
+        values = synthetic.make_b(k, n, seed=100 + replay, kind="int").cuda()
+        b.copy_(values)
+        d.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = torch.empty_like(d)
+        _native.matmul_prepared(prep, values, eager, m, n, k)
+        torch.cuda.synchronize()
+        assert torch.equal(d, eager)
+        assert bool(torch.isfinite(d).all())
+
+
 def test_reference_benchmark_dataset():
     """tests/kernel_test.cu:302-306,398-400: all value bits 1, all metadata 0x4444 => rows t % 4 < 2 of B summed."""
     m, n, k = 256, 128, 512
