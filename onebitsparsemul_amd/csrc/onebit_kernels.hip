@@ -941,9 +941,28 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   }
   u32x4_t breg[8];
   AChunk a_cur[R], a_next[R];
-  if (kPrefetchB) load_b(wave * kChunkK, breg);
-  load_a(wave, a_cur);
-  for (int kc = wave; kc < kc_total; kc += NW) {
+  // Short K (at most two chunks per wavefront, e.g. 11008 x 4096): everything the wavefront will read is requested
+  // at once, so the kernel pays one memory latency instead of one per chunk.
+  constexpr bool kShortPath = NW <= 8 && SUB == 1 && MODE != kSkinnyBScalar;
+  const bool short_k = kShortPath && kc_total <= 2 * NW;
+  if (short_k) {
+    u32x4_t breg2[8];
+    load_b(wave * kChunkK, breg);
+    load_a(wave, a_cur);
+    load_b((wave + NW) * kChunkK, breg2);  // all zeros when the wavefront has one chunk only
+    load_a(wave + NW, a_next);
+    if (wave < kc_total) {
+      store_b(wave * kChunkK, breg);
+      compute(a_cur, std::integral_constant<int, 0>{});
+    }
+    if (wave + NW < kc_total) {
+      store_b((wave + NW) * kChunkK, breg2);
+      compute(a_next, std::integral_constant<int, 0>{});
+    }
+  }
+  if (kPrefetchB && !short_k) load_b(wave * kChunkK, breg);
+  if (!short_k) load_a(wave, a_cur);
+  for (int kc = short_k ? kc_total : wave; kc < kc_total; kc += NW) {
     const int k_base = kc * kChunkK;
     if (!kPrefetchB) load_b(k_base, breg);
     store_b(k_base, breg);  // after the previous image's fragment reads: LDS operations of a wavefront execute in order
