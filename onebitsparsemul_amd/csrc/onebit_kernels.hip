@@ -41,35 +41,35 @@ __global__ __launch_bounds__(64) void prepare_kernel(const uint8_t* __restrict__
       else
         word = (uint32_t)src[0] | ((uint32_t)src[1] << 8) | ((uint32_t)src[2] << 16) | ((uint32_t)src[3] << 24);
     }
-    column_bits[local] = word;
+    column_bits[local] = ~word;  // stored inverted: a set bit now means -1, which is what the sign words hold
   }
   __syncthreads();
   uint32_t meta[4] = {0, 0, 0, 0};
   uint32_t sign[2] = {0, 0};
+  // metadata column of step s: c = 16 kc + 2 s + ga. In all three layouts the element of column c + 2 lies a fixed
+  // distance after that of column c (one column pair = 2 m elements in the reordered layouts), so one offset is
+  // computed and then advanced.
+  const int c0 = kc * 16 + ga;
+  int64_t off = layout == 0 ? meta_offset_reference(r, c0, m) : layout == 1 ? meta_offset_cutlass(r, c0, m) : r * ncols + c0;
+  const int64_t off_step = layout == 2 ? 2 : 2 * (int64_t)m;
 #pragma unroll
   for (int s = 0; s < kStepsPerChunk; ++s) {
-    const int c = kc * 16 + 2 * s + ga;
+    const int c = c0 + 2 * s;
     uint32_t mv = 0x4444u;
-    if (c < ncols) {
-      int64_t off;
-      if (layout == 0) off = meta_offset_reference(r, c, m);
-      else if (layout == 1) off = meta_offset_cutlass(r, c, m);
-      else off = r * ncols + c;
-      mv = e[off];
-    }
+    if (c < ncols) mv = e[off];
+    off += off_step;
     meta[s >> 1] |= mv << (16 * (s & 1));
-    // kept value t of this step = compressed column 8 c + t = entry 8 (2 s + ga) + t of the block's 128
+    // kept value t of this step = compressed column 8 c + t = entry 8 (2 s + ga) + t of the block's 128; it goes to
+    // bit 15 - j (t even) or 31 - j (t odd) of the step group's sign word, j = 4 (s % 4) + t / 2: one bit-field
+    // extract and one shift-or per value
     const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(&column_bits[8 * (2 * s + ga)]);
     const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(&column_bits[8 * (2 * s + ga) + 4]);
     const uint32_t w8[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    uint32_t neg = 0;  // bit t set: kept value t of this step is -1
 #pragma unroll
-    for (int t = 0; t < 8; ++t) neg |= (((w8[t] >> i) & 1u) ^ 1u) << t;
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-      const int j = 4 * (s & 3) + p;
-      sign[s >> 2] |= ((neg >> (2 * p)) & 1u) << (15 - j);
-      sign[s >> 2] |= ((neg >> (2 * p + 1)) & 1u) << (31 - j);
+    for (int t = 0; t < 8; ++t) {
+      const int j = 4 * (s & 3) + (t >> 1);
+      const int position = ((t & 1) ? 31 : 15) - j;
+      sign[s >> 2] |= ((w8[t] >> i) & 1u) << position;
     }
   }
   uint8_t* block = prep + ((size_t)rb * kc_total + kc) * kBlockBytes;
