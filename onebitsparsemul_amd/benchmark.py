@@ -3,6 +3,7 @@ README.md:23-26, script/cuda_run_test.sh):
 
     python -m onebitsparsemul_amd.benchmark --a_rows=8192 --n=8192 --a_cols=8192 --reference-check=false
     python -m onebitsparsemul_amd.benchmark --sweep            # 512 ... 12800 squares, 30 iterations each
+    python -m onebitsparsemul_amd.benchmark --sweep --json sweep.json --csv sweep.csv
 
 Prints the reference's table columns (a_rows, n, a_cols, GFLOPs = 2*M*N*K / t, runtime in ms). Timing mirrors
 tests/kernel_test.cu:619-691: one warm-up, then `iterations` back-to-back launches between two events. Output
@@ -62,6 +63,8 @@ def main(argv=None):
     ap.add_argument("--reference-check", dest="reference_check", type=_bool, default=False)
     ap.add_argument("--fp16-out", action="store_true", help="fp16 C/D instead of the reference's fp32")
     ap.add_argument("--sweep", action="store_true", help="the reference's square sweep, 30 iterations each")
+    ap.add_argument("--json", default=None, metavar="PATH", help="also write the rows as a JSON list to PATH")
+    ap.add_argument("--csv", default=None, metavar="PATH", help="also write the rows as CSV to PATH")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
         sys.exit("this benchmark needs a GPU")
@@ -71,6 +74,7 @@ def main(argv=None):
     print("| a_rows |   n   | a_cols |    GFLOPs    | Runtime (ms) |" + (" check |" if args.reference_check else ""))
     print("|--------|-------|--------|--------------|--------------|" + ("-------|" if args.reference_check else ""))
     ok = True
+    rows = []
     for (m, n, k) in shapes:
         ms, gflops, passed = run(m, n, k, args.alpha, args.beta, iterations, args.reference_check, dtype)
         line = f"| {m:6d} | {n:5d} | {k:6d} | {gflops:12.1f} | {ms:12.6f} |"
@@ -78,6 +82,18 @@ def main(argv=None):
             line += " Passed |" if passed else " FAILED |"
             ok = ok and passed
         print(line, flush=True)
+        rows.append(dict(a_rows=m, n=n, a_cols=k, gflops=gflops, runtime_ms=ms, alpha=args.alpha, beta=args.beta,
+                         iterations=iterations, out_dtype="fp16" if args.fp16_out else "fp32", check=passed))
+    if args.json:
+        import json
+        with open(args.json, "w") as fh:
+            json.dump(rows, fh, indent=1)
+    if args.csv:
+        import csv
+        with open(args.csv, "w", newline="") as fh:
+            writer = csv.DictWriter(fh, fieldnames=list(rows[0].keys()))
+            writer.writeheader()
+            writer.writerows(rows)
     return 0 if ok else 1
 
 

@@ -502,6 +502,20 @@ def test_benchmark_cli_reference_check():
                            "--iterations=2", "--fp16-out"]) == 0
 
 
+def test_benchmark_cli_writes_json_and_csv(tmp_path):
+    import csv
+    import json
+    from onebitsparsemul_amd import benchmark
+    js, cs = tmp_path / "rows.json", tmp_path / "rows.csv"
+    assert benchmark.main(["--a_rows=256", "--n=64", "--a_cols=256", "--reference-check=true", "--iterations=1",
+                           f"--json={js}", f"--csv={cs}"]) == 0
+    rows = json.loads(js.read_text())
+    assert len(rows) == 1 and rows[0]["a_rows"] == 256 and rows[0]["check"] is True and rows[0]["gflops"] > 0
+    with open(cs) as fh:
+        table = list(csv.DictReader(fh))
+    assert len(table) == 1 and table[0]["a_cols"] == "256"
+
+
 @pytest.mark.parametrize("prune", [True, False])
 def test_gpu_packer_matches_host_pipeline(prune):
     """onebit_sparse_pack (fused HIP kernel) against the oracle's mask + compress + quantise + pack, ties included."""
