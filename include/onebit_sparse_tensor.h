@@ -104,6 +104,12 @@ void onebit_sparse_set_split_k(int splits);
  * kernel's element-copy variant reads B in place (much slower; always used when k * n < 65536). */
 void onebit_sparse_set_pad_b(int enabled);
 
+/* Diagnostic, no counterpart in the reference, host-only (touches no GPU): what a prepared call of this shape would
+ * launch under the current hooks. plan[0] = 1 for the split-K kernel (n <= 64), 0 for the main kernel; plan[1] =
+ * weight rows per workgroup (split-K kernel) or the tile code (main kernel); plan[2] = K splits over workgroups
+ * (main kernel, 1 = none); plan[3] = 1 if B is read through a padded copy. */
+int onebit_sparse_describe_launch(int m, int n, int k, int b_16_byte_aligned, int *plan);
+
 /* Diagnostic, no counterpart in the reference: sustained rate of v_smfmac_f32_32x32x32_f16 in a register-only
  * loop on the current device (one wavefront per SIMD, `iterations` x 16 instructions each), in dense-equivalent
  * TFLOP/s. random_operands = 1 uses +-1 values, N(0,1) fp16 B values and random 2:4 indices (the benchmark's

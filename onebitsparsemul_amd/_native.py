@@ -15,7 +15,7 @@ META_REFERENCE, META_CUTLASS, META_LOGICAL = 0, 1, 2
 EXPORTS = (
     "onebit_sparse_matmul", "onebit_sparse_matmul_ex", "onebit_sparse_prepared_bytes", "onebit_sparse_prepare",
     "onebit_sparse_matmul_prepared", "onebit_sparse_pack", "onebit_sparse_last_error", "onebit_sparse_set_tile_config",
-    "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_set_split_k", "onebit_sparse_set_pad_b",
+    "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_set_split_k", "onebit_sparse_set_pad_b", "onebit_sparse_describe_launch",
     "onebit_sparse_measure_smfmac_rate", "onebit_sparse_device_info",
 )
 
@@ -53,6 +53,8 @@ def lib():
         L.onebit_sparse_set_split_k.argtypes = [i32]
         L.onebit_sparse_set_pad_b.restype = None
         L.onebit_sparse_set_pad_b.argtypes = [i32]
+        L.onebit_sparse_describe_launch.restype = i32
+        L.onebit_sparse_describe_launch.argtypes = [i32, i32, i32, i32, ctypes.POINTER(ctypes.c_int)]
         L.onebit_sparse_device_info.restype = i32
         L.onebit_sparse_device_info.argtypes = [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
         L.onebit_sparse_measure_smfmac_rate.restype = i32
@@ -194,3 +196,12 @@ def device_info():
     cus, khz = ctypes.c_int(0), ctypes.c_int(0)
     _check(lib().onebit_sparse_device_info(ctypes.byref(cus), ctypes.byref(khz)))
     return cus.value, khz.value
+
+
+def describe_launch(m, n, k, b_aligned=True):
+    """What a prepared call of this shape would launch (host-only): dict(kernel, rows or tile, splits, pad_b)."""
+    plan = (ctypes.c_int * 4)()
+    _check(lib().onebit_sparse_describe_launch(m, n, k, 1 if b_aligned else 0, plan))
+    if plan[0]:
+        return dict(kernel="skinny_kernel", rows=plan[1])
+    return dict(kernel="gemm_kernel", tile=plan[1], splits=plan[2], pad_b=bool(plan[3]))

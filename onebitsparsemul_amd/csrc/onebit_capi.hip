@@ -159,16 +159,47 @@ GemmPlan plan_gemm(int m, int n, int k) {
   return best;
 }
 
+// Everything the C ABI decides about one prepared call, from the shape and the alignment of B alone (no GPU needed).
+struct LaunchPlan {
+  int split_k_kernel;  // 1: skinny_kernel, 0: gemm_kernel
+  int rows_or_tile;    // skinny_kernel: weight rows per workgroup; gemm_kernel: TileConfig
+  int splits;          // gemm_kernel: K splits over workgroups (1 = none)
+  int pad_b;           // gemm_kernel: B is read through a padded copy
+};
+
+LaunchPlan choose_launch(int m, int n, int k, bool b_16_byte_aligned) {
+  LaunchPlan plan{};
+  // 32 < n <= 64: every 32-row workgroup of the split-K kernel stages all of B, which the main kernel's tiles
+  // overtake from about 16k rows on (28672 x 64 x 8192: 43 us against 58 us; 11008 x 64 x 4096: 21 against 17)
+  const bool skinny_shape = n <= 32 || (n <= onebit::kSkinnyMaxN && m <= 16384);
+  if (skinny_shape && g_skinny_enabled.load()) {
+    int rows = g_skinny_rows.load();
+    // the largest row group that still gives about two workgroups per three compute units (measured: larger groups
+    // re-read B less often, but idle compute units cost more)
+    if (rows <= 0) rows = n > 32 ? 32 : (m / 128 >= 160 && n <= 16) ? 128 : (m / 64 >= 160) ? 64 : 32;
+    plan.split_k_kernel = 1;
+    plan.rows_or_tile = rows;
+    plan.splits = 1;
+    return plan;
+  }
+  const GemmPlan gemm = plan_gemm(m, n, k);
+  plan.rows_or_tile = gemm.tile;
+  plan.splits = gemm.splits;
+  // B rows that are not 16-byte aligned: pad a copy (one extra pass over B) unless the problem is too small for that
+  // to pay against the element-copy variant of the kernel
+  const bool b_in_place = n % 8 == 0 && b_16_byte_aligned;
+  plan.pad_b = !b_in_place && (size_t)k * n >= 65536 && g_pad_b.load();
+  return plan;
+}
+
 int matmul_prepared_impl(const void* prepared, const void* b, const void* c, void* d, int m, int n, int k, float alpha,
                          float beta, int c_dtype, int d_dtype, hipStream_t stream) {
   if (!prepared || !b || !d) return fail(ONEBIT_ERR_ARGUMENT, "null operand pointer");
   if (beta != 0.f && !c) return fail(ONEBIT_ERR_ARGUMENT, "c must not be null when beta != 0");
   const int kc_total = (k + onebit::kChunkK - 1) / onebit::kChunkK;
 
-  // 32 < n <= 64: every 32-row workgroup of the split-K kernel stages all of B, which the main kernel's tiles
-  // overtake from about 16k rows on (28672 x 64 x 8192: 43 us against 58 us; 11008 x 64 x 4096: 21 against 17)
-  const bool skinny_shape = n <= 32 || (n <= onebit::kSkinnyMaxN && m <= 16384);
-  if (skinny_shape && g_skinny_enabled.load()) {
+  const LaunchPlan plan = choose_launch(m, n, k, (reinterpret_cast<uintptr_t>(b) & 15) == 0);
+  if (plan.split_k_kernel) {
     onebit::SkinnyArgs args{};
     args.prep = static_cast<const uint8_t*>(prepared);
     args.b = static_cast<const _Float16*>(b);
@@ -179,11 +210,7 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
     args.alpha = alpha; args.beta = beta;
     args.c_f16 = c_dtype == ONEBIT_DTYPE_F16;
     args.d_f16 = d_dtype == ONEBIT_DTYPE_F16;
-    int rows = g_skinny_rows.load();
-    // the largest row group that still gives about two workgroups per three compute units (measured: larger groups
-    // re-read B less often, but idle compute units cost more)
-    if (rows <= 0) rows = n > 32 ? 32 : (m / 128 >= 160 && n <= 16) ? 128 : (m / 64 >= 160) ? 64 : 32;
-    ONEBIT_HIP(onebit::launch_skinny(args, rows, stream));
+    ONEBIT_HIP(onebit::launch_skinny(args, plan.rows_or_tile, stream));
     return ONEBIT_OK;
   }
 
@@ -197,13 +224,9 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
   args.alpha = alpha; args.beta = beta;
   args.c_f16 = c_dtype == ONEBIT_DTYPE_F16;
   args.d_f16 = d_dtype == ONEBIT_DTYPE_F16;
-  const GemmPlan plan = plan_gemm(m, n, k);
-  const int tile = plan.tile;
+  const int tile = plan.rows_or_tile;
   const int splits = plan.splits;
-  // B rows that are not 16-byte aligned: pad a copy (one extra pass over B) unless the problem is too small for that
-  // to pay against the element-copy variant of the kernel
-  const bool b_in_place = n % 8 == 0 && (reinterpret_cast<uintptr_t>(b) & 15) == 0;
-  const bool pad_b = !b_in_place && (size_t)k * n >= 65536 && g_pad_b.load();
+  const bool pad_b = plan.pad_b != 0;
   if (splits > 1 || pad_b) {
     int device = 0;
     ONEBIT_HIP(hipGetDevice(&device));
@@ -242,6 +265,18 @@ void onebit_sparse_set_skinny_enabled(int enabled) { g_skinny_enabled.store(enab
 void onebit_sparse_set_skinny_rows(int rows) { g_skinny_rows.store(rows); }
 void onebit_sparse_set_split_k(int splits) { g_split_k.store(splits); }
 void onebit_sparse_set_pad_b(int enabled) { g_pad_b.store(enabled ? 1 : 0); }
+
+int onebit_sparse_describe_launch(int m, int n, int k, int b_16_byte_aligned, int* plan) {
+  g_last_error.clear();
+  if (!plan) return fail(ONEBIT_ERR_ARGUMENT, "plan must not be null");
+  if (int rc = check_shape(m, n, k)) return rc;
+  const LaunchPlan p = choose_launch(m, n, k, b_16_byte_aligned != 0);
+  plan[0] = p.split_k_kernel;
+  plan[1] = p.rows_or_tile;
+  plan[2] = p.splits;
+  plan[3] = p.pad_b;
+  return ONEBIT_OK;
+}
 
 size_t onebit_sparse_prepared_bytes(int m, int k) {
   if (m <= 0 || k <= 0) return 0;

@@ -106,3 +106,72 @@ def test_binding_module_loads_and_validates():
     c = torch.zeros(64, 8, dtype=torch.float32)
     with pytest.raises(RuntimeError):
         onebit_sparse_cuda.onebit_mul(a, b, meta, c)  # host tensors are rejected, nothing is computed on the CPU
+
+
+@pytest.fixture
+def _default_hooks():
+    def reset():
+        _native.set_tile_config(-1)
+        _native.set_skinny_enabled(True)
+        _native.set_skinny_rows(-1)
+        _native.set_split_k(-1)
+        _native.set_pad_b(True)
+    reset()
+    yield
+    reset()
+
+
+def test_launch_plan_of_the_benchmark_shapes(_default_hooks):
+    """kernel choice of the C ABI (host logic, no GPU): the five benchmark configurations and the cases around them"""
+    plan = _native.describe_launch
+    # large squares: 512 x 128 tile on eight wavefronts (code 9), one pass, B read in place
+    for size in (4096, 8192, 16384, 25600):
+        assert plan(size, size, size) == dict(kernel="gemm_kernel", tile=9, splits=1, pad_b=False)
+    # a last round of 512 x 128 tiles that would be mostly empty: 256 x 128 on four wavefronts (code 4)
+    assert plan(6144, 6144, 6144)["tile"] == 4 and plan(11008, 2048, 4096)["tile"] == 4
+    # the prefill shape has one 256 x 128 tile per CU: its eight-wavefront form (code 10)
+    assert plan(4096, 2048, 4096) == dict(kernel="gemm_kernel", tile=10, splits=1, pad_b=False)
+    # small squares: 128 x 128 / 64 x 128 tiles, no K split
+    assert plan(2048, 2048, 2048) == dict(kernel="gemm_kernel", tile=11, splits=1, pad_b=False)
+    assert plan(512, 512, 512) == dict(kernel="gemm_kernel", tile=12, splits=1, pad_b=False)
+    # decode shapes: the split-K kernel, row group by M
+    for n in (1, 4, 16):
+        assert plan(11008, n, 4096) == dict(kernel="skinny_kernel", rows=64)
+        assert plan(4096, n, 11008) == dict(kernel="skinny_kernel", rows=32)
+    assert plan(28672, 16, 8192) == dict(kernel="skinny_kernel", rows=128)
+    assert plan(28672, 32, 8192) == dict(kernel="skinny_kernel", rows=64)
+    assert plan(11008, 64, 4096) == dict(kernel="skinny_kernel", rows=32)
+    assert plan(28672, 64, 8192)["kernel"] == "gemm_kernel"      # from 16k rows on the main kernel is faster
+    assert plan(4096, 65, 4096)["kernel"] == "gemm_kernel"
+    # few tiles over a long K: split over workgroups; many tiles: never
+    few = plan(4096, 128, 4096)
+    assert few["kernel"] == "gemm_kernel" and few["splits"] > 1
+    assert plan(4096, 256, 11008)["splits"] > 1
+    # B rows that are not 16-byte aligned: padded copy, except for tiny operands
+    assert plan(4096, 1001, 4096)["pad_b"] is True
+    assert plan(4096, 1000, 4096, b_aligned=False)["pad_b"] is True
+    assert plan(4096, 1000, 4096)["pad_b"] is False
+    assert plan(256, 72, 128, b_aligned=False)["pad_b"] is False
+
+
+def test_launch_plan_follows_the_hooks(_default_hooks):
+    plan = _native.describe_launch
+    _native.set_skinny_enabled(False)
+    assert plan(11008, 16, 4096)["kernel"] == "gemm_kernel"
+    _native.set_skinny_enabled(True)
+    _native.set_skinny_rows(32)
+    assert plan(28672, 16, 8192) == dict(kernel="skinny_kernel", rows=32)
+    _native.set_tile_config(4)
+    _native.set_split_k(3)
+    assert plan(8192, 8192, 8192) == dict(kernel="gemm_kernel", tile=4, splits=3, pad_b=False)
+    _native.set_split_k(1000)
+    assert plan(8192, 8192, 8192)["splits"] == 32          # at most one split per 256 of K
+    _native.set_pad_b(False)
+    assert plan(4096, 1001, 4096)["pad_b"] is False
+
+
+def test_describe_launch_validates():
+    lib = _native.lib()
+    out = (ctypes.c_int * 4)()
+    assert lib.onebit_sparse_describe_launch(60, 8, 32, 1, out) == 1
+    assert lib.onebit_sparse_describe_launch(64, 8, 32, 1, None) == 1
