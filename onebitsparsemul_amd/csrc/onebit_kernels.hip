@@ -86,69 +86,79 @@ __global__ __launch_bounds__(64) void prepare_kernel(const uint8_t* __restrict__
 // pruned first), compression to kept values + nibbles (:126-159, including the fixed encodings of groups
 // with fewer or more than two non-zeros), sign quantisation (value > 0 -> 1, __init__.py:22-23), transposed
 // bit packing (__init__.py:25-34,142-143) and the metadata reorder (:21-48).
-// One wavefront = 64 consecutive rows x one metadata column (16 dense K); the eight sign bits of a row are
-// gathered across the wavefront with ballots, so every store of `a` is 8 bytes of 64 consecutive rows.
+// One wavefront = 64 consecutive rows x four metadata columns (64 dense K, one 128-byte line per row); the eight
+// sign bits of a row and column are gathered across the wavefront with ballots, so every store of `a` is 8 bytes
+// of 64 consecutive rows.
 // =====================================================================================================
 __device__ __constant__ uint8_t kNibbleOfPattern[16] = {0xE, 0x8, 0x9, 0x4, 0xE, 0x8, 0x9, 0x4,
                                                         0xE, 0xC, 0xD, 0x4, 0xE, 0xC, 0xD, 0x4};
 
 __global__ __launch_bounds__(64) void pack_kernel(const _Float16* __restrict__ w, uint8_t* __restrict__ a,
                                                   uint16_t* __restrict__ e, int m, int k, int prune, int layout) {
-  const int c = blockIdx.x;                         // metadata column
   const int64_t r = (int64_t)blockIdx.y * 64 + threadIdx.x;  // m % 64 == 0: always a valid row
   const int ncols = k / 16;
-  u32x4_t raw[2];
-  const u32x4_t* src = reinterpret_cast<const u32x4_t*>(w + r * k + 16 * c);
-  raw[0] = src[0];
-  raw[1] = src[1];
-  _Float16 v[16];
-  __builtin_memcpy(v, raw, 32);
-  uint32_t word = 0, bits = 0;  // bits: bit t = kept value t of this metadata element is > 0
+  // four metadata columns (64 weights = 128 consecutive bytes of the lane's row) per wavefront: requests of whole
+  // 128-byte lines; the last group of a row may hold two columns only (k % 32 == 0)
+  const int c_first = blockIdx.x * 4;
+  const int c_count = ncols - c_first < 4 ? ncols - c_first : 4;
+  u32x4_t line[8];
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    float x[4], mag[4];
+  for (int i = 0; i < 8; ++i)
+    if (i < 2 * c_count) line[i] = reinterpret_cast<const u32x4_t*>(w + r * k + 16 * c_first)[i];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      x[i] = (float)v[4 * g + i];
-      mag[i] = x[i] < 0.f ? -x[i] : x[i];
-    }
-    int pattern = 0;
+  for (int ci = 0; ci < 4; ++ci) {
+    if (ci >= c_count) break;  // wave-uniform
+    const int c = c_first + ci;                       // metadata column
+    u32x4_t raw[2] = {line[2 * ci], line[2 * ci + 1]};
+    _Float16 v[16];
+    __builtin_memcpy(v, raw, 32);
+    uint32_t word = 0, bits = 0;  // bits: bit t = kept value t of this metadata element is > 0
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      bool keep = true;
-      if (prune) {
-        int beaten = 0;  // elements that outrank i: larger magnitude, or equal magnitude and higher index
+    for (int g = 0; g < 4; ++g) {
+      float x[4], mag[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) beaten += (j != i) && (mag[j] > mag[i] || (mag[j] == mag[i] && j > i));
-        keep = beaten < 2;
+      for (int i = 0; i < 4; ++i) {
+        x[i] = (float)v[4 * g + i];
+        mag[i] = x[i] < 0.f ? -x[i] : x[i];
       }
-      if (!keep) x[i] = 0.f;
-      pattern |= (x[i] != 0.f) << i;
-    }
-    const int nib = kNibbleOfPattern[pattern];
-    const int i0 = nib & 3, i1 = nib >> 2;
-    word |= (uint32_t)nib << (4 * g);
-    float k0 = x[0], k1 = x[0];
+      int pattern = 0;
 #pragma unroll
-    for (int i = 1; i < 4; ++i) {
-      if (i0 == i) k0 = x[i];
-      if (i1 == i) k1 = x[i];
-    }
-    bits |= (uint32_t)(k0 > 0.f) << (2 * g);
-    bits |= (uint32_t)(k1 > 0.f) << (2 * g + 1);
-  }
-  int64_t off;
-  if (layout == 0) off = meta_offset_reference(r, c, m);
-  else if (layout == 1) off = meta_offset_cutlass(r, c, m);
-  else off = r * ncols + c;
-  e[off] = (uint16_t)word;
-  const int64_t row0 = (int64_t)blockIdx.y * 64;
+      for (int i = 0; i < 4; ++i) {
+        bool keep = true;
+        if (prune) {
+          int beaten = 0;  // elements that outrank i: larger magnitude, or equal magnitude and higher index
 #pragma unroll
-  for (int t = 0; t < 8; ++t) {
-    const uint64_t mask = __ballot((bits >> t) & 1u);  // bit l = row row0 + l, compressed column 8c + t
-    if (threadIdx.x == 0) {
-      const int64_t pos = row0 + (int64_t)(8 * c + t) * m;  // multiple of 64
-      *reinterpret_cast<uint64_t*>(a + (pos >> 3)) = mask;
+          for (int j = 0; j < 4; ++j) beaten += (j != i) && (mag[j] > mag[i] || (mag[j] == mag[i] && j > i));
+          keep = beaten < 2;
+        }
+        if (!keep) x[i] = 0.f;
+        pattern |= (x[i] != 0.f) << i;
+      }
+      const int nib = kNibbleOfPattern[pattern];
+      const int i0 = nib & 3, i1 = nib >> 2;
+      word |= (uint32_t)nib << (4 * g);
+      float k0 = x[0], k1 = x[0];
+#pragma unroll
+      for (int i = 1; i < 4; ++i) {
+        if (i0 == i) k0 = x[i];
+        if (i1 == i) k1 = x[i];
+      }
+      bits |= (uint32_t)(k0 > 0.f) << (2 * g);
+      bits |= (uint32_t)(k1 > 0.f) << (2 * g + 1);
+    }
+    int64_t off;
+    if (layout == 0) off = meta_offset_reference(r, c, m);
+    else if (layout == 1) off = meta_offset_cutlass(r, c, m);
+    else off = r * ncols + c;
+    e[off] = (uint16_t)word;
+    const int64_t row0 = (int64_t)blockIdx.y * 64;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const uint64_t mask = __ballot((bits >> t) & 1u);  // bit l = row row0 + l, compressed column 8c + t
+      if (threadIdx.x == 0) {
+        const int64_t pos = row0 + (int64_t)(8 * c + t) * m;  // multiple of 64
+        *reinterpret_cast<uint64_t*>(a + (pos >> 3)) = mask;
+      }
     }
   }
 }
@@ -1111,7 +1121,7 @@ hipError_t launch_prepare(const void* a, const void* e, void* prep, int m, int k
 }
 
 hipError_t launch_pack(const void* w, void* a, void* e, int m, int k, int prune, int layout, hipStream_t stream) {
-  hipLaunchKernelGGL(pack_kernel, dim3(k / 16, m / 64), dim3(64), 0, stream, (const _Float16*)w, (uint8_t*)a,
+  hipLaunchKernelGGL(pack_kernel, dim3((k / 16 + 3) / 4, m / 64), dim3(64), 0, stream, (const _Float16*)w, (uint8_t*)a,
                      (uint16_t*)e, m, k, prune, layout);
   return hipGetLastError();
 }
