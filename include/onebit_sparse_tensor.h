@@ -104,6 +104,17 @@ void onebit_sparse_set_split_k(int splits);
  * kernel's element-copy variant reads B in place (much slower; always used when k * n < 65536). */
 void onebit_sparse_set_pad_b(int enabled);
 
+/* Opt-in cache for callers of the one-call entry points (onebit_sparse_matmul, onebit_sparse_matmul_ex) whose
+ * weights do not change, which is inference: with entries > 0 the library keeps the reordered copy of up to that
+ * many weights per device, keyed by (a, e, m, k, meta_layout), in its own device memory, and a call with a known
+ * key skips the reorder kernel (decode 11008 x 4096 x 16: one kernel instead of two). The caller promises that the
+ * memory at a and e is neither modified nor freed and reused while its entry exists; after changing or freeing
+ * weights call onebit_sparse_clear_weight_cache(). entries <= 0 (the default, the reference's behaviour: nothing is
+ * retained between calls) switches the cache off and clears it. Least recently used entries are evicted (with a
+ * device synchronization). A first use allocates with hipMalloc: not inside a stream capture. */
+int onebit_sparse_set_weight_cache(int entries);
+int onebit_sparse_clear_weight_cache(void);
+
 /* Diagnostic, no counterpart in the reference, host-only (touches no GPU): what a prepared call of this shape would
  * launch under the current hooks. plan[0] = 1 for the split-K kernel (n <= 64), 0 for the main kernel; plan[1] =
  * weight rows per workgroup (split-K kernel) or the tile code (main kernel); plan[2] = K splits over workgroups

@@ -19,7 +19,7 @@ from ._semi_structured_conversions import (
 __all__ = [
     "cuda_binary_mul", "cuda_binary_mul_", "binary_quant", "pack_binary", "unpack_binary", "dequant_desparse_tile",
     "py_binary_gemm", "BinaryLinear_2_4", "PreparedWeight", "mask_creator", "sparse_semi_structured_from_dense_cutlass",
-    "sparse_semi_structured_to_dense_cutlass",
+    "sparse_semi_structured_to_dense_cutlass", "set_weight_cache", "clear_weight_cache",
 ]
 
 
@@ -27,6 +27,17 @@ def _binding():
     """The compiled torch binding `onebit_sparse_cuda` (reference: onebit_sparse_mul/torch_kernel_cuda.cpp)."""
     from . import onebit_sparse_cuda  # noqa: PLC0415  (compiled module, built in-tree)
     return onebit_sparse_cuda
+
+
+def set_weight_cache(entries):
+    """Let `cuda_binary_mul` / `onebit_mul` / the C entry points keep the reordered copy of up to `entries` weights
+    per GPU, keyed by the weight tensors' addresses (0, the default, keeps nothing: the reference's behaviour).
+    Only for weights that are neither modified nor freed while cached; see include/onebit_sparse_tensor.h."""
+    _native.set_weight_cache(entries)
+
+
+def clear_weight_cache():
+    _native.clear_weight_cache()
 
 
 def _problem_shape(A, B, meta):

@@ -15,7 +15,7 @@ META_REFERENCE, META_CUTLASS, META_LOGICAL = 0, 1, 2
 EXPORTS = (
     "onebit_sparse_matmul", "onebit_sparse_matmul_ex", "onebit_sparse_prepared_bytes", "onebit_sparse_prepare",
     "onebit_sparse_matmul_prepared", "onebit_sparse_pack", "onebit_sparse_last_error", "onebit_sparse_set_tile_config",
-    "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_set_split_k", "onebit_sparse_set_pad_b", "onebit_sparse_describe_launch",
+    "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_set_split_k", "onebit_sparse_set_pad_b", "onebit_sparse_describe_launch", "onebit_sparse_set_weight_cache", "onebit_sparse_clear_weight_cache",
     "onebit_sparse_measure_smfmac_rate", "onebit_sparse_device_info",
 )
 
@@ -53,6 +53,10 @@ def lib():
         L.onebit_sparse_set_split_k.argtypes = [i32]
         L.onebit_sparse_set_pad_b.restype = None
         L.onebit_sparse_set_pad_b.argtypes = [i32]
+        L.onebit_sparse_set_weight_cache.restype = i32
+        L.onebit_sparse_set_weight_cache.argtypes = [i32]
+        L.onebit_sparse_clear_weight_cache.restype = i32
+        L.onebit_sparse_clear_weight_cache.argtypes = []
         L.onebit_sparse_describe_launch.restype = i32
         L.onebit_sparse_describe_launch.argtypes = [i32, i32, i32, i32, ctypes.POINTER(ctypes.c_int)]
         L.onebit_sparse_device_info.restype = i32
@@ -205,3 +209,12 @@ def describe_launch(m, n, k, b_aligned=True):
     if plan[0]:
         return dict(kernel="skinny_kernel", rows=plan[1])
     return dict(kernel="gemm_kernel", tile=plan[1], splits=plan[2], pad_b=bool(plan[3]))
+
+
+def set_weight_cache(entries):
+    """Opt-in cache of reordered weights for the one-call entry points (0 = off, the default)."""
+    _check(lib().onebit_sparse_set_weight_cache(entries))
+
+
+def clear_weight_cache():
+    _check(lib().onebit_sparse_clear_weight_cache())

@@ -12,6 +12,7 @@
 #include <map>
 #include <mutex>
 #include <string>
+#include <vector>
 
 namespace {
 
@@ -21,6 +22,7 @@ std::atomic<int> g_skinny_enabled{1};
 std::atomic<int> g_skinny_rows{-1};
 std::atomic<int> g_split_k{-1};
 std::atomic<int> g_pad_b{1};
+std::atomic<int> g_weight_cache_entries{0};
 
 int fail(int code, const char* fmt, ...) {
   char buf[512];
@@ -56,6 +58,18 @@ struct DeviceState {
   std::map<hipStream_t, Buffer> split_ws;
   // B with rows padded to a multiple of 8 columns (operands the asynchronous copies cannot read in place), per stream
   std::map<hipStream_t, Buffer> b_pad;
+  // opt-in cache of prepared operands of the one-call entry points, keyed by the caller's weight pointers
+  struct CachedWeight {
+    const void* a;
+    const void* e;
+    int m, k, layout;
+    void* prep;
+    hipStream_t stream;  // the stream its reorder kernel was enqueued on
+    hipEvent_t ready;    // recorded after that kernel
+    unsigned long last_use;
+  };
+  std::vector<CachedWeight> weight_cache;
+  unsigned long use_counter = 0;
 };
 DeviceState g_dev[kMaxDevices];
 
@@ -330,6 +344,46 @@ int onebit_sparse_matmul_ex(const void* a, const void* b, const void* c, void* d
   if (device < 0 || device >= kMaxDevices) return fail(ONEBIT_ERR_HIP, "device index %d out of range", device);
   DeviceState& ds = g_dev[device];
   void* prep = nullptr;
+  const int cache_entries = g_weight_cache_entries.load();
+  if (cache_entries > 0) {
+    {  // the lock ends before the multiplication is launched, which may take it again for its own buffers
+      std::lock_guard<std::mutex> lock(ds.mu);
+      for (auto& w : ds.weight_cache)
+        if (w.a == a && w.e == e && w.m == m && w.k == k && w.layout == meta_layout) {
+          w.last_use = ++ds.use_counter;
+          if (w.stream != s) ONEBIT_HIP(hipStreamWaitEvent(s, w.ready, 0));  // its reorder kernel ran on another stream
+          prep = w.prep;
+          break;
+        }
+      if (!prep) {
+        if ((int)ds.weight_cache.size() >= cache_entries) {  // evict the least recently used entry
+          size_t victim = 0;
+          for (size_t i = 1; i < ds.weight_cache.size(); ++i)
+            if (ds.weight_cache[i].last_use < ds.weight_cache[victim].last_use) victim = i;
+          ONEBIT_HIP(hipDeviceSynchronize());  // earlier work on any stream may still read it
+          ONEBIT_HIP(hipFree(ds.weight_cache[victim].prep));
+          ONEBIT_HIP(hipEventDestroy(ds.weight_cache[victim].ready));
+          ds.weight_cache.erase(ds.weight_cache.begin() + victim);
+        }
+        DeviceState::CachedWeight w{a, e, m, k, meta_layout, nullptr, s, nullptr, ++ds.use_counter};
+        ONEBIT_HIP(hipMalloc(&w.prep, onebit::prepared_bytes(m, k)));
+        if (hipError_t st = hipEventCreateWithFlags(&w.ready, hipEventDisableTiming); st != hipSuccess) {
+          (void)hipFree(w.prep);
+          return fail(ONEBIT_ERR_HIP, "HIP error '%s' from hipEventCreateWithFlags", hipGetErrorString(st));
+        }
+        hipError_t st = onebit::launch_prepare(a, e, w.prep, m, k, meta_layout, s);
+        if (st == hipSuccess) st = hipEventRecord(w.ready, s);
+        if (st != hipSuccess) {
+          (void)hipFree(w.prep);
+          (void)hipEventDestroy(w.ready);
+          return fail(ONEBIT_ERR_HIP, "HIP error '%s' while reordering a cached weight", hipGetErrorString(st));
+        }
+        ds.weight_cache.push_back(w);
+        prep = w.prep;
+      }
+    }
+    return matmul_prepared_impl(prep, b, c, d, m, n, k, alpha, beta, c_dtype, d_dtype, s);
+  }
   {
     std::lock_guard<std::mutex> lock(ds.mu);
     if (int rc = grow(&ds.prep, &ds.prep_bytes, onebit::prepared_bytes(m, k))) return rc;
@@ -337,6 +391,34 @@ int onebit_sparse_matmul_ex(const void* a, const void* b, const void* c, void* d
   }
   ONEBIT_HIP(onebit::launch_prepare(a, e, prep, m, k, meta_layout, s));
   return matmul_prepared_impl(prep, b, c, d, m, n, k, alpha, beta, c_dtype, d_dtype, s);
+}
+
+int onebit_sparse_clear_weight_cache(void) {
+  g_last_error.clear();
+  int previous = 0;
+  const bool have_device = hipGetDevice(&previous) == hipSuccess;
+  int rc = ONEBIT_OK;
+  for (int device = 0; device < kMaxDevices; ++device) {
+    DeviceState& ds = g_dev[device];
+    std::lock_guard<std::mutex> lock(ds.mu);
+    if (ds.weight_cache.empty()) continue;
+    if (hipSetDevice(device) != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
+      rc = fail(ONEBIT_ERR_HIP, "cannot synchronize device %d to clear its weight cache", device);
+      continue;
+    }
+    for (auto& w : ds.weight_cache) {
+      (void)hipFree(w.prep);
+      (void)hipEventDestroy(w.ready);
+    }
+    ds.weight_cache.clear();
+  }
+  if (have_device) (void)hipSetDevice(previous);
+  return rc;
+}
+
+int onebit_sparse_set_weight_cache(int entries) {
+  g_weight_cache_entries.store(entries > 0 ? entries : 0);
+  return entries > 0 ? ONEBIT_OK : onebit_sparse_clear_weight_cache();
 }
 
 void onebit_sparse_matmul(void* a, void* b, void* c, void* d, void* e, int m, int n, int k) {

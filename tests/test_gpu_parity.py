@@ -27,12 +27,14 @@ def _defaults():
     _native.set_skinny_rows(-1)
     _native.set_split_k(-1)
     _native.set_pad_b(True)
+    _native.set_weight_cache(0)
     yield
     _native.set_tile_config(-1)
     _native.set_skinny_enabled(True)
     _native.set_skinny_rows(-1)
     _native.set_split_k(-1)
     _native.set_pad_b(True)
+    _native.set_weight_cache(0)
 
 
 def _gpu(*ts):
@@ -428,6 +430,47 @@ def test_hip_graph_replays_match_eager(m, n, k):
         torch.cuda.synchronize()
         assert torch.equal(d, eager)
         assert bool(torch.isfinite(d).all())
+
+
+def test_weight_cache_of_the_one_call_entry_points():
+    """opt-in cache keyed by the weight pointers: a hit skips the reorder kernel (so a weight changed in place
+    keeps giving the old result until the cache is cleared), least-recently-used eviction, use from a second stream,
+    and the default (off) re-reads the weight on every call"""
+    m, n, k = 256, 16, 512
+    weights = []
+    for seed in (1, 2, 3):
+        a, meta = synthetic.make_weight(m, k, seed=seed)
+        weights.append((a.cuda(), meta.cuda(), oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)))
+    bi = synthetic.make_b(k, n, seed=7, kind="int")
+    bd = bi.cuda()
+
+    def run(a, meta):
+        d = torch.empty((m, n), dtype=torch.float32, device="cuda")
+        _native.matmul_ex(a, bd, meta, d, m, n, k)
+        torch.cuda.synchronize()
+        return d.cpu().numpy()
+
+    want = [oracle.host_gemm(dense, bi.numpy(), d_dtype=oracle.F32, acc="f32") for _, _, dense in weights]
+    _native.set_weight_cache(2)
+    for _ in range(2):                                    # miss, then hit
+        assert np.array_equal(run(weights[0][0], weights[0][1]), want[0])
+    assert np.array_equal(run(weights[1][0], weights[1][1]), want[1])
+    assert np.array_equal(run(weights[2][0], weights[2][1]), want[2])   # evicts weight 0
+    assert np.array_equal(run(weights[0][0], weights[0][1]), want[0])   # miss again, evicts weight 1
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):                         # a hit from another stream waits for the reorder kernel
+        assert np.array_equal(run(weights[0][0], weights[0][1]), want[0])
+    # the cache really is used: flip the stored signs in place, the cached copy still gives the old result
+    a0 = weights[0][0]
+    a0.copy_(a0 ^ 0xFF)
+    torch.cuda.synchronize()
+    assert np.array_equal(run(a0, weights[0][1]), want[0])
+    _native.clear_weight_cache()
+    assert np.array_equal(run(a0, weights[0][1]), -want[0])
+    _native.set_weight_cache(0)                           # default: nothing is retained between calls
+    a0.copy_(a0 ^ 0xFF)
+    torch.cuda.synchronize()
+    assert np.array_equal(run(a0, weights[0][1]), want[0])
 
 
 def test_reference_benchmark_dataset():
