@@ -57,8 +57,9 @@ void onebit_sparse_matmul(void *a, void *b, void *c, void *d, void *e, int m, in
  * hard-codes at :60-62 and the dtypes of csrc/kernel.h:17-18 turned into arguments): alpha/beta epilogue
  * (csrc/kernel.h:27-31), fp16 or fp32 c and d, metadata layout, explicit stream (hipStream_t passed as
  * void*, NULL = default stream). Returns a status code and never exits.
- * The reordered copy of (a, e) is written to a library-owned per-device workspace on every call, so calls
- * that overlap on different streams of one device must use the prepared form below instead.
+ * The reordered copy of (a, e) is written on every call to a library-owned workspace kept per device and per
+ * stream (grown with a device synchronization when a larger weight arrives): calls on different streams may
+ * overlap; the prepared form below skips the reorder pass and allocates nothing.
  */
 int onebit_sparse_matmul_ex(const void *a, const void *b, const void *c, void *d, const void *e, int m, int n, int k,
                             float alpha, float beta, int c_dtype, int d_dtype, int meta_layout, void *stream);

@@ -43,16 +43,16 @@ int fail(int code, const char* fmt, ...) {
 
 constexpr int kMaxDevices = 64;
 
-// Library-owned device memory: the reordered operand of the one-call entry points. Grow-only, one per
-// device, freed at process exit by the runtime. Work that uses it is ordered by the caller's stream.
+// Library-owned device memory. Grow-only, one buffer per device and stream (calls on one stream are ordered, calls
+// on different streams must not share a buffer), freed at process exit by the runtime.
 struct Buffer {
   void* ptr = nullptr;
   size_t bytes = 0;
 };
 struct DeviceState {
   std::mutex mu;
-  void* prep = nullptr;
-  size_t prep_bytes = 0;
+  // the reordered operand of the one-call entry points (when the weight cache is off)
+  std::map<hipStream_t, Buffer> prep;
   // fp32 partial sums of the K-split passes: one buffer per stream, so that calls on different streams do not
   // share one (calls on the same stream are ordered)
   std::map<hipStream_t, Buffer> split_ws;
@@ -386,8 +386,9 @@ int onebit_sparse_matmul_ex(const void* a, const void* b, const void* c, void* d
   }
   {
     std::lock_guard<std::mutex> lock(ds.mu);
-    if (int rc = grow(&ds.prep, &ds.prep_bytes, onebit::prepared_bytes(m, k))) return rc;
-    prep = ds.prep;
+    Buffer& own = ds.prep[s];
+    if (int rc = grow(&own.ptr, &own.bytes, onebit::prepared_bytes(m, k))) return rc;
+    prep = own.ptr;
   }
   ONEBIT_HIP(onebit::launch_prepare(a, e, prep, m, k, meta_layout, s));
   return matmul_prepared_impl(prep, b, c, d, m, n, k, alpha, beta, c_dtype, d_dtype, s);

@@ -6,6 +6,7 @@
 // csrc/warp.h:18-690) with code written for 64-wide wavefronts; nothing is translated from them.
 #include "onebit_device.h"
 #include "onebit_launch.h"
+#include <atomic>
 #include <type_traits>
 
 namespace onebit {
@@ -1133,16 +1134,16 @@ static hipError_t launch_gemm_cfg(GemmArgs args, hipStream_t stream) {
   args.tiles_n = (args.n + TS::BN - 1) / TS::BN;
   const int lds = DMA ? TS::LDS_BYTES : TS::STAGE_BYTES;
   auto kern = gemm_kernel<WM, WN, FM, FN, DMA>;
-  // the dynamic-LDS limit is a per-device attribute of the kernel; racing writers store the same value
-  static bool attr_done[64] = {};
+  // the dynamic-LDS limit is a per-device attribute of the kernel; threads that race here set the same value
+  static std::atomic<bool> attr_done[64] = {};
   int device = 0;
   if (hipError_t st = hipGetDevice(&device); st != hipSuccess) return st;
   if (device < 0 || device >= 64) return hipErrorInvalidDevice;
-  if (!attr_done[device]) {
+  if (!attr_done[device].load(std::memory_order_acquire)) {
     hipError_t st = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (st != hipSuccess) return st;
-    attr_done[device] = true;
+    attr_done[device].store(true, std::memory_order_release);
   }
   hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, args.splits), dim3(64 * TS::NW), lds, stream, args);
   return hipGetLastError();

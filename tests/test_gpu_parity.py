@@ -264,6 +264,27 @@ def test_k_split_streams_do_not_share_partial_sums():
         assert np.array_equal(o.cpu().numpy(), oracle.host_gemm(dense, b.cpu().numpy(), d_dtype=oracle.F32, acc="f32"))
 
 
+def test_one_call_entry_point_on_several_streams_keeps_the_reordered_weights_apart():
+    """the one-call entry point reorders the weight into a library buffer on every call: calls on different streams
+    with different weights must not share that buffer"""
+    m, n, k = 512, 256, 4096
+    weights = [synthetic.make_weight(m, k, seed=70 + i) for i in range(3)]
+    dev = [_gpu(a, meta) for a, meta in weights]
+    b = synthetic.make_b(k, n, seed=75, kind="int")
+    bd = b.cuda()
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    outs = [torch.empty((m, n), dtype=torch.float32, device="cuda") for _ in range(3)]
+    torch.cuda.synchronize()
+    for _ in range(20):
+        for s, (ad, md), o in zip(streams, dev, outs):
+            with torch.cuda.stream(s):
+                _native.matmul_ex(ad, bd, md, o, m, n, k)
+    torch.cuda.synchronize()
+    for (a, meta), o in zip(weights, outs):
+        dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
+        assert np.array_equal(o.cpu().numpy(), oracle.host_gemm(dense, b.numpy(), d_dtype=oracle.F32, acc="f32"))
+
+
 def test_config3_split_k_is_deterministic_and_reusable():
     m, k, n = 4096, 11008, 16
     a, meta = synthetic.make_weight(m, k, seed=5)
