@@ -76,6 +76,17 @@ int onebit_sparse_matmul_prepared(const void *prepared, const void *b, const voi
                                   float alpha, float beta, int c_dtype, int d_dtype, void *stream);
 
 /*
+ * Linear-layer form of the prepared product, for the forward pass of BinaryLinear_2_4
+ * (onebit_sparse_mul/__init__.py:116-128), whose activations are token-major:
+ *     y[t][r] = sum over k of W[r][k] * x[t][k]  (+ bias[r] when bias is not NULL)
+ * x: fp16, tokens x k, row-major, 16-byte aligned; y: tokens x m, row-major, fp16 or fp32 (y_dtype); bias: m values,
+ * fp16 or fp32 (bias_dtype), or NULL. Same result as onebit_sparse_matmul_prepared on B = transpose(x) followed by
+ * a transpose of D and the bias addition, without those passes: the kernels read x and write y where they lie.
+ */
+int onebit_sparse_linear_prepared(const void *prepared, const void *x, const void *bias, void *y, int tokens, int m,
+                                  int k, int bias_dtype, int y_dtype, void *stream);
+
+/*
  * Packs a dense fp16 weight (m x k, row-major, device) into the stored operands a (m*k/16 bytes) and e
  * (m*k/8 bytes) on the GPU. Replaces the tensor-op pipeline of BinaryLinear_2_4.pack
  * (onebit_sparse_mul/__init__.py:130-145 with _semi_structured_conversions.py:54-179,286-314): prune != 0 first

@@ -122,6 +122,14 @@ class PreparedWeight:
             out = torch.empty((self.m, n), dtype=out_dtype, device=b.device)
         return _native.matmul_prepared(self.buffer, b, out, self.m, n, self.k, c=c, alpha=alpha, beta=beta)
 
+    def linear(self, x, bias=None, out=None, out_dtype=torch.float16):
+        """y (tokens, m) = x (tokens, k) @ W.T (+ bias): the layer's form, x and y token-major, no transposes."""
+        if x.data_ptr() % 16:
+            x = x.clone()  # a view that starts inside a 16-byte unit
+        if out is None:
+            out = torch.empty((x.shape[0], self.m), dtype=out_dtype, device=x.device)
+        return _native.linear_prepared(self.buffer, x, out, self.m, self.k, bias=bias)
+
 
 class BinaryLinear_2_4(nn.Module):
     """1-bit 2:4 sparse linear layer: y = x @ W.T (+ bias when one has been assigned), W (outfeatures, infeatures)
@@ -171,9 +179,10 @@ class BinaryLinear_2_4(nn.Module):
         if self._prepared is None or self._prepared.buffer.device != x.device:
             self._prepared = PreparedWeight(self.packed_binary_sparse.to(x.device), self.meta.to(x.device))
         lead = x.shape[:-1]
-        b = x.reshape(-1, self.infeatures).to(torch.float16).T.contiguous()  # (k, batch)
-        out = self._prepared.matmul(b, out_dtype=torch.float16)           # (outfeatures, batch)
-        y = out.T.reshape(*lead, self.outfeatures).to(x.dtype)
-        if self.bias is not None:
-            y = y + self.bias.to(y.dtype)
-        return y
+        tokens = x.reshape(-1, self.infeatures).to(torch.float16).contiguous()
+        bias = self.bias
+        if bias is not None and (bias.dtype not in (torch.float16, torch.float32) or bias.device != x.device):
+            bias = bias.to(device=x.device, dtype=torch.float32)
+        # one kernel: reads the tokens where they lie, adds the bias, writes (tokens, outfeatures)
+        y = self._prepared.linear(tokens, bias=bias.contiguous() if bias is not None else None)
+        return y.reshape(*lead, self.outfeatures).to(x.dtype)

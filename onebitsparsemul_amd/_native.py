@@ -14,7 +14,7 @@ META_REFERENCE, META_CUTLASS, META_LOGICAL = 0, 1, 2
 
 EXPORTS = (
     "onebit_sparse_matmul", "onebit_sparse_matmul_ex", "onebit_sparse_prepared_bytes", "onebit_sparse_prepare",
-    "onebit_sparse_matmul_prepared", "onebit_sparse_pack", "onebit_sparse_last_error", "onebit_sparse_set_tile_config",
+    "onebit_sparse_matmul_prepared", "onebit_sparse_linear_prepared", "onebit_sparse_pack", "onebit_sparse_last_error", "onebit_sparse_set_tile_config",
     "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_set_split_k", "onebit_sparse_set_pad_b", "onebit_sparse_describe_launch", "onebit_sparse_set_weight_cache", "onebit_sparse_clear_weight_cache",
     "onebit_sparse_measure_smfmac_rate", "onebit_sparse_device_info",
 )
@@ -39,6 +39,8 @@ def lib():
         L.onebit_sparse_prepare.argtypes = [vp, vp, i32, i32, i32, vp, vp]
         L.onebit_sparse_matmul_prepared.restype = i32
         L.onebit_sparse_matmul_prepared.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, i32, vp]
+        L.onebit_sparse_linear_prepared.restype = i32
+        L.onebit_sparse_linear_prepared.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp]
         L.onebit_sparse_pack.restype = i32
         L.onebit_sparse_pack.argtypes = [vp, i32, i32, i32, vp, vp, i32, vp]
         L.onebit_sparse_last_error.restype = ctypes.c_char_p
@@ -131,6 +133,23 @@ def matmul_prepared(prepared, b, d, m, n, k, c=None, alpha=1.0, beta=0.0):
             prepared.data_ptr(), b.data_ptr(), c.data_ptr() if c is not None else None, d.data_ptr(), m, n, k,
             alpha, beta, _dtype_code(c) if c is not None else F32, _dtype_code(d), _stream(b)))
     return d
+
+
+def linear_prepared(prepared, x, y, m, k, bias=None):
+    """y (tokens, m) = x (tokens, k) @ W.T (+ bias), x fp16 and y fp16 / fp32, both token-major and contiguous."""
+    dev = _require_cuda(prepared, x, y, bias)
+    tokens = x.shape[0]
+    if x.dtype != torch.float16 or tuple(x.shape) != (tokens, k):
+        raise ValueError("x must be float16 of shape (tokens, k)")
+    if tuple(y.shape) != (tokens, m) or (bias is not None and tuple(bias.shape) != (m,)):
+        raise ValueError("y must have shape (tokens, m) and bias (m,)")
+    if prepared.numel() != prepared_bytes(m, k):
+        raise ValueError("prepared operand does not match m, k")
+    with torch.cuda.device(dev):
+        _check(lib().onebit_sparse_linear_prepared(
+            prepared.data_ptr(), x.data_ptr(), bias.data_ptr() if bias is not None else None, y.data_ptr(), tokens, m, k,
+            _dtype_code(bias) if bias is not None else F16, _dtype_code(y), _stream(x)))
+    return y
 
 
 def matmul_ex(a, b, meta, d, m, n, k, c=None, alpha=1.0, beta=0.0, layout=META_REFERENCE):

@@ -329,6 +329,65 @@ int onebit_sparse_matmul_prepared(const void* prepared, const void* b, const voi
   return matmul_prepared_impl(prepared, b, c, d, m, n, k, alpha, beta, c_dtype, d_dtype, static_cast<hipStream_t>(stream));
 }
 
+int onebit_sparse_linear_prepared(const void* prepared, const void* x, const void* bias, void* y, int tokens, int m,
+                                  int k, int bias_dtype, int y_dtype, void* stream) {
+  g_last_error.clear();
+  if (int rc = check_shape(m, tokens, k)) return rc;
+  if (int rc = check_dtype(bias_dtype, y_dtype)) return rc;
+  if (!prepared || !x || !y) return fail(ONEBIT_ERR_ARGUMENT, "null operand pointer");
+  if ((reinterpret_cast<uintptr_t>(x) & 15) != 0) return fail(ONEBIT_ERR_ARGUMENT, "x must be 16-byte aligned");
+  const int kc_total = (k + onebit::kChunkK - 1) / onebit::kChunkK;
+  const LaunchPlan plan = choose_launch(m, tokens, k, true);
+  if (plan.split_k_kernel) {
+    onebit::SkinnyArgs args{};
+    args.prep = static_cast<const uint8_t*>(prepared);
+    args.b = static_cast<const _Float16*>(x);
+    args.d = y;
+    args.m = m; args.n = tokens; args.k = k;
+    args.kc_total = kc_total;
+    args.alpha = 1.f; args.beta = 0.f;
+    args.d_f16 = y_dtype == ONEBIT_DTYPE_F16;
+    args.bias = bias;
+    args.bias_f16 = bias_dtype == ONEBIT_DTYPE_F16;
+    ONEBIT_HIP(onebit::launch_skinny_tokens(args, plan.rows_or_tile, static_cast<hipStream_t>(stream)));
+    return ONEBIT_OK;
+  }
+  switch (plan.rows_or_tile) {
+    case onebit::kTile256x128w: case onebit::kTile128x128s: case onebit::kTile512x128w8: case onebit::kTile256x128w8:
+    case onebit::kTile128x128w8: case onebit::kTile64x128: break;
+    default:
+      return fail(ONEBIT_ERR_ARGUMENT, "tile configuration %d has no token-major variant (4, 6, 9, 10, 11, 12 have)",
+                  plan.rows_or_tile);
+  }
+  onebit::GemmArgs args{};
+  args.prep = static_cast<const uint8_t*>(prepared);
+  args.b = static_cast<const _Float16*>(x);
+  args.d = y;
+  args.m = m; args.n = tokens; args.k = k;
+  args.kc_total = kc_total;
+  args.d_f16 = y_dtype == ONEBIT_DTYPE_F16;
+  args.bias = bias;
+  args.bias_f16 = bias_dtype == ONEBIT_DTYPE_F16;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (plan.splits > 1) {
+    int device = 0;
+    ONEBIT_HIP(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) return fail(ONEBIT_ERR_ARGUMENT, "device ordinal %d not supported", device);
+    DeviceState& st = g_dev[device];
+    std::lock_guard<std::mutex> lock(st.mu);
+    const int cps = (kc_total + plan.splits - 1) / plan.splits;
+    args.chunks_per_split = cps;
+    args.splits = (kc_total + cps - 1) / cps;  // every split non-empty
+    Buffer& ws = st.split_ws[s];
+    if (int rc = grow(&ws.ptr, &ws.bytes, (size_t)args.splits * m * tokens * sizeof(float)); rc != ONEBIT_OK) return rc;
+    args.split_ws = static_cast<float*>(ws.ptr);
+    ONEBIT_HIP(onebit::launch_gemm_tokens(args, plan.rows_or_tile, s));
+    return ONEBIT_OK;
+  }
+  ONEBIT_HIP(onebit::launch_gemm_tokens(args, plan.rows_or_tile, s));
+  return ONEBIT_OK;
+}
+
 int onebit_sparse_matmul_ex(const void* a, const void* b, const void* c, void* d, const void* e, int m, int n, int k,
                             float alpha, float beta, int c_dtype, int d_dtype, int meta_layout, void* stream) {
   g_last_error.clear();

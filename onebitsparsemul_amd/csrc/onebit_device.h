@@ -21,6 +21,7 @@
 
 namespace onebit {
 
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half16_t __attribute__((ext_vector_type(16)));
 typedef float float16_t __attribute__((ext_vector_type(16)));

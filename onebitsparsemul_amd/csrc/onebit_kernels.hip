@@ -320,6 +320,32 @@ __device__ __forceinline__ void load_b_frags(const char* stage_lds, int ks, half
   }
 }
 
+// Token-major stage image (linear-layer form): row t = the stage's 64 K values of token t (128 bytes, eight 16-byte
+// pieces, piece p stored at position p ^ token_swizzle(t)). The operand of K step ks is pieces 4 ks + gb and 4 ks + 2 + gb of
+// the lane's token: two plain 16-byte reads at the precomputed lane offsets piece_off[2 ks + h].
+// Position XOR of the 16-byte pieces of token row t in the token-major images: sixteen consecutive tokens that read the
+// same piece touch sixteen different 16-byte columns of the 256 bytes the LDS banks span (rows of 128 bytes: two rows
+// fill the span, so the XOR changes every second token; rows of 256 bytes or more: every token).
+template <int ROW_BYTES = 128>
+__device__ __forceinline__ constexpr int token_swizzle(int token) {
+  return ROW_BYTES >= 256 ? (token & 15) : ((token >> 1) & 7);
+}
+
+template <int FN>
+__device__ __forceinline__ void load_b_frags_tokens(const char* wave_lds, int ks, half16_t (&bv)[FN],
+                                                    const int (&piece_off)[4]) {
+#pragma unroll
+  for (int fn = 0; fn < FN; ++fn) {
+    u32x8_t raw;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const u32x4_t t = *reinterpret_cast<const u32x4_t*>(wave_lds + piece_off[2 * ks + h] + fn * (32 * kStageK * 2));
+      raw[4 * h] = t.x; raw[4 * h + 1] = t.y; raw[4 * h + 2] = t.z; raw[4 * h + 3] = t.w;
+    }
+    bv[fn] = __builtin_bit_cast(half16_t, raw);
+  }
+}
+
 template <int STEP, int FM>
 __device__ __forceinline__ void expand_frags(const AChunk (&a)[FM], uint32_t one, half8_t (&av)[FM]) {
   if (ONEBIT_EXP_NO_EXPAND) {
@@ -382,8 +408,11 @@ __device__ __forceinline__ void interleave_region() {
 // Source of zeros for the asynchronous copies of B rows at or past K.
 __device__ __attribute__((aligned(16))) uint32_t g_zero16[4] = {0, 0, 0, 0};
 
-template <int WM, int WN, int FM, int FN, bool DMA>
+// TOKENS (with DMA only): the linear-layer form. p.b is x (p.n tokens x p.k, token-major), p.d is y (p.n tokens x
+// p.m), the epilogue is y = acc + bias; a tile column is a token.
+template <int WM, int WN, int FM, int FN, bool DMA, bool TOKENS = false>
 __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmArgs p) {
+  static_assert(DMA || !TOKENS, "the token-major form uses the asynchronous copies");
   using TS = TileShape<WM, WN, FM, FN>;
   constexpr int BM = TS::BM, BN = TS::BN, CH = TS::CH, NL = TS::NL, NW = TS::NW;
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -420,6 +449,19 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
     frag_off[fn] = ((lc ^ chunk_swizzle<BN>(lane_row)) << 4) + (c8 & 1) * 8;
   }
 
+  int piece_off[4];  // token-major image: byte offsets of the lane's four pieces of a stage (see load_b_frags_tokens)
+  {
+    const int token = lane & 31;
+    const int base = token * (kStageK * 2) + ((gb ^ token_swizzle(token)) << 4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) piece_off[j] = base ^ ((4 * (j >> 1) + 2 * (j & 1)) << 4);
+  }
+  const char* const wave_image = smem + wn * FN * (32 * kStageK * 2);  // first token row of this wavefront in stage 0
+  auto read_frags = [&](int ring_slot, int ks, half16_t (&bv)[FN]) __attribute__((always_inline)) {
+    if constexpr (TOKENS) load_b_frags_tokens<FN>(wave_image + ring_slot * TS::STAGE_BYTES, ks, bv, piece_off);
+    else load_b_frags<FN, BN>(smem + ring_slot * TS::STAGE_BYTES, ks, bv, frag_off, lane_row_off);
+  };
+
   const uint32_t one = packed_one_in_vgpr();
   float16_t acc[FM][FN];
 #pragma unroll
@@ -441,22 +483,31 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
     // copy i of wavefront w fills LDS slots [(NW i + w) * 64, +64) of the stage; slot = (row, physical chunk).
     // Global address = wave-uniform base of the stage + per-lane byte offset.
     uint32_t b_off[NL];
-    int copy_row[NL];
+    int copy_row[NL];  // first K row of the stage that copy i carries
     uint32_t lds_dst[NL];
     const uint32_t smem_base = lds_offset_of(smem);
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
       const int slot = (NW * i + wave) * 64 + lane;
-      const int row = slot / CH, pc = slot % CH;
-      const int lc = pc ^ chunk_swizzle<BN>(row);
-      int col = 8 * lc;
-      if (n0 + col >= p.ldb) col = 0;  // columns past the row: any valid address will do, the results are not stored
-      b_off[i] = (uint32_t)(row * p.ldb + col) * 2u;
-      copy_row[i] = row;
+      if constexpr (TOKENS) {
+        // slot = (token of the tile, physical piece): fetches K values [8 lc, 8 lc + 8) of the stage for that token
+        int token = slot / 8;
+        const int lc = (slot % 8) ^ token_swizzle(token);
+        if (n0 + token >= p.n) token = 0;  // tokens past the end: any valid address will do, the results are not stored
+        b_off[i] = (uint32_t)(token * p.k + 8 * lc) * 2u;  // the launcher checks that BN * k * 2 fits 32 bits
+        copy_row[i] = 8 * lc;
+      } else {
+        const int row = slot / CH, pc = slot % CH;
+        const int lc = pc ^ chunk_swizzle<BN>(row);
+        int col = 8 * lc;
+        if (n0 + col >= p.ldb) col = 0;  // columns past the row: any valid address will do, the results are not stored
+        b_off[i] = (uint32_t)(row * p.ldb + col) * 2u;
+        copy_row[i] = row;
+      }
       lds_dst[i] = smem_base + (NW * i + wave) * 1024;
     }
-    const size_t stage_stride = (size_t)kStageK * p.ldb * 2;
-    const char* b_stage = reinterpret_cast<const char*>(p.b) + (size_t)n0 * 2 +
+    const size_t stage_stride = TOKENS ? (size_t)kStageK * 2 : (size_t)kStageK * p.ldb * 2;
+    const char* b_stage = reinterpret_cast<const char*>(p.b) + (TOKENS ? (size_t)n0 * p.k * 2 : (size_t)n0 * 2) +
                           (size_t)chunk_begin * kStages * stage_stride;  // advances one stage per copy
     const char* zeros = reinterpret_cast<const char*>(g_zero16);
     int next_k0 = chunk_begin * kChunkK;  // first K row of the next stage to copy
@@ -533,12 +584,12 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
     __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm) a_cur[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);
-    load_b_frags<FN, BN>(smem, 0, bv0, frag_off, lane_row_off);
+    read_frags(0, 0, bv0);
     expand_frags<0>(a_cur, one, av0);
 
 #define ONEBIT_STAGE(S, WAITCNT, ISSUE_A)                                                                        \
     {                                                                                                            \
-      load_b_frags<FN, BN>(smem + (S) * TS::STAGE_BYTES, 1, bv1, frag_off, lane_row_off);                         \
+      read_frags((S), 1, bv1);                                                                                   \
       expand_frags<2 * (S) + 1>(a_cur, one, av1);                                                                \
       mfma_frags<2 * (S)>(a_cur, av0, bv0, acc);                                                                 \
       interleave_region<FM, FN>();                                                                               \
@@ -547,7 +598,7 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
       if (!ONEBIT_EXP_NO_BARRIER) __builtin_amdgcn_s_barrier();                                                  \
       if (ISSUE_A) issue_a();                                                                                    \
       issue_b(S);                                                                                                \
-      load_b_frags<FN, BN>(smem + (((S) + 1) % kStages) * TS::STAGE_BYTES, 0, bv0, frag_off, lane_row_off);       \
+      read_frags(((S) + 1) % kStages, 0, bv0);                                                                   \
     }
 
     for (int kc = chunk_begin; kc < chunk_end; ++kc) {
@@ -611,6 +662,109 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
   }
 
   smfmac_drain();
+  if constexpr (TOKENS) {
+    // ---- epilogue of the linear-layer form: y[token][row] = acc + bias[row], fp16 (RNE) or fp32 ----
+    const int token_lane = lane & 31;
+    auto bias_of = [&](int row) __attribute__((always_inline)) {
+      if (!p.bias) return 0.f;
+      return p.bias_f16 ? (float)reinterpret_cast<const _Float16*>(p.bias)[row] : reinterpret_cast<const float*>(p.bias)[row];
+    };
+    // COUNT (4 or 8) consecutive bias values starting at a row that is a multiple of COUNT, by 16-byte loads
+    auto bias_vector = [&](int row, float* out, auto count_tag) __attribute__((always_inline)) {
+      constexpr int COUNT = decltype(count_tag)::value;
+#pragma unroll
+      for (int e = 0; e < COUNT; ++e) out[e] = 0.f;
+      if (!p.bias) return;
+      if (p.bias_f16) {
+        if constexpr (COUNT == 8) {
+          const half8_t v = *reinterpret_cast<const half8_t*>(reinterpret_cast<const _Float16*>(p.bias) + row);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) out[e] = (float)v[e];
+        } else {
+          const half4_t v = *reinterpret_cast<const half4_t*>(reinterpret_cast<const _Float16*>(p.bias) + row);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) out[e] = (float)v[e];
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < COUNT; e += 4) {
+          const float4 v = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.bias) + row + e);
+          out[e] = v.x; out[e + 1] = v.y; out[e + 2] = v.z; out[e + 3] = v.w;
+        }
+      }
+    };
+    if (p.vector_epilogue) {
+      // Each wavefront turns one 32-row block of its tile at a time through a private LDS scratch laid out
+      // [token][32 rows] fp32: a lane's four accumulator registers of one group are four consecutive rows of its token,
+      // one 16-byte slot (slot s = rows 4 s ... 4 s + 3, stored at position s ^ (token % 8) against bank conflicts);
+      // then every lane handles 16 bytes of one token's row of y.
+      __syncthreads();  // every wavefront is done with the stage ring, which becomes the scratch
+      constexpr int WCOLS = FN * 32;
+      char* scratch = smem + wave * (WCOLS * 128);
+#pragma unroll
+      for (int fm = 0; fm < FM; ++fm) {
+#pragma unroll
+        for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            *reinterpret_cast<float4*>(scratch + (fn * 32 + token_lane) * 128 + (((2 * q + gb) ^ token_swizzle(token_lane)) << 4)) =
+                float4{acc[fm][fn][4 * q], acc[fm][fn][4 * q + 1], acc[fm][fn][4 * q + 2], acc[fm][fn][4 * q + 3]};
+        const int row_base = row0 + fm * 32;
+        if (p.d_f16) {
+#pragma unroll
+          for (int it = 0; it < WCOLS * 4 / 64; ++it) {
+            const int piece = it * 64 + lane;
+            const int t = piece / 4, j = piece % 4;
+            const int token = col0 + t, row = row_base + 8 * j;
+            const float4 lo = *reinterpret_cast<const float4*>(scratch + t * 128 + (((2 * j) ^ token_swizzle(t)) << 4));
+            const float4 hi = *reinterpret_cast<const float4*>(scratch + t * 128 + (((2 * j + 1) ^ token_swizzle(t)) << 4));
+            const float x[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            if (token < p.n && row < p.m) {
+              float bias8[8];
+              bias_vector(row, bias8, std::integral_constant<int, 8>{});
+              half8_t out;
+#pragma unroll
+              for (int e = 0; e < 8; ++e) out[e] = (_Float16)(x[e] + bias8[e]);
+              *reinterpret_cast<half8_t*>(reinterpret_cast<_Float16*>(d_out) + (size_t)token * p.m + row) = out;
+            }
+          }
+        } else {
+#pragma unroll
+          for (int it = 0; it < WCOLS * 8 / 64; ++it) {
+            const int piece = it * 64 + lane;
+            const int t = piece / 8, j = piece % 8;
+            const int token = col0 + t, row = row_base + 4 * j;
+            const float4 v4 = *reinterpret_cast<const float4*>(scratch + t * 128 + ((j ^ token_swizzle(t)) << 4));
+            if (token < p.n && row < p.m) {
+              float bias4[4];
+              bias_vector(row, bias4, std::integral_constant<int, 4>{});
+              *reinterpret_cast<float4*>(reinterpret_cast<float*>(d_out) + (size_t)token * p.m + row) =
+                  float4{v4.x + bias4[0], v4.y + bias4[1], v4.z + bias4[2], v4.w + bias4[3]};
+            }
+          }
+        }
+      }
+      return;
+    }
+    // y not 16-byte aligned: one element per accumulator register
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+      for (int fn = 0; fn < FN; ++fn) {
+        const int token = col0 + fn * 32 + token_lane;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int row = row0 + fm * 32 + 8 * (v / 4) + 4 * gb + (v % 4);
+          if (token < p.n && row < p.m) {
+            const float x = acc[fm][fn][v] + bias_of(row);
+            const size_t o = (size_t)token * p.m + row;
+            if (p.d_f16) reinterpret_cast<_Float16*>(d_out)[o] = (_Float16)x;
+            else reinterpret_cast<float*>(d_out)[o] = x;
+          }
+        }
+      }
+    return;
+  }
   // ---- epilogue: D = alpha * acc + beta * C (csrc/kernel.h:27-31), fp16 (RNE) or fp32 output ----
   if constexpr (DMA) {
     if (p.vector_epilogue) {
@@ -740,7 +894,12 @@ constexpr int kSkinnyRegion = 8192;  // bytes of one B image
 
 // how B rows reach the image: whole rows are the image rows (n == NC), rows of n % 8 == 0 elements in 16-byte
 // pieces padded to the image row, 8-byte rows (n == 4, NC == 16), or element by element (any n <= NC, any alignment)
-enum SkinnyBMode { kSkinnyBFull = 0, kSkinnyB8 = 1, kSkinnyB4 = 2, kSkinnyBScalar = 3 };
+// kSkinnyBTokens: the token-major form of the linear layer. B is x, n rows (tokens) of k consecutive values, and
+// the result is written as y[token][weight row] (+ bias[weight row]). The image is then token-major too: row t holds
+// the image's K range of token t in 16-byte pieces, piece p stored at position p ^ token_swizzle(t) so that lanes
+// which read the same piece of consecutive tokens fall into different banks; a lane's SMFMAC operand is two plain
+// 16-byte reads (K consecutive inside a piece), no transpose.
+enum SkinnyBMode { kSkinnyBFull = 0, kSkinnyB8 = 1, kSkinnyB4 = 2, kSkinnyBScalar = 3, kSkinnyBTokens = 4 };
 
 // 16-byte piece q of the image whose first row is B row k_base: image row q / (NC / 8), columns 8 (q % (NC / 8))
 // ... + 7; zero outside B. Vector modes only.
@@ -782,6 +941,10 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   static_assert(NC == 16 || NC == 32 || NC == 64, "image width");
   static_assert(MODE != kSkinnyB4 || NC == 16, "the 8-byte-row mode is for 16 columns");
   static_assert(R * TILE_BYTES <= kSkinnyRegion, "partial tiles reuse the wavefront's image memory");
+  constexpr bool TOKENS = MODE == kSkinnyBTokens;
+  constexpr int PPT = IMG_ROWS / 8;                    // token-major image: 16-byte pieces per token row
+  constexpr int TPI = 64 / PPT;                        // ... and tokens covered by the 64 pieces of one wavefront load
+  constexpr int TOKEN_ROW_BYTES = IMG_ROWS * 2;
   __shared__ __attribute__((aligned(16))) char bs[NW * kSkinnyRegion];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -828,8 +991,23 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   // Image t of this wavefront = B rows [k_base, k_base + IMG_ROWS) with k_base = (wave + NW (t / SUB)) * 256 +
   // (t % SUB) * IMG_ROWS. Vector modes: the image travels through registers, loaded while the previous image is
   // multiplied; element mode: loaded and stored in one go when the image is due.
+  // token-major image: piece lane + 64 i = K values [8 p, 8 p + 8) of the image for token token_lane + TPI i
+  const int piece_lane = lane % PPT, token_lane = lane / PPT;
+  const uint32_t token_load_base = ((uint32_t)token_lane * (uint32_t)k_rows + 8u * piece_lane) * 2u;
+  const uint32_t token_load_step = (uint32_t)TPI * (uint32_t)k_rows * 2u;
+  const uint32_t token_store_base =
+      (uint32_t)token_lane * TOKEN_ROW_BYTES + (uint32_t)((piece_lane ^ token_swizzle<TOKEN_ROW_BYTES>(token_lane)) << 4);
   auto load_b = [&](int k_base, u32x4_t (&v)[8]) __attribute__((always_inline)) {
     if (MODE == kSkinnyBScalar) return;
+    if (TOKENS) {
+      // offsets at or past n * k * 2 (tokens >= n) fall outside the descriptor and read as zero; K positions at or
+      // past k are sent there too (the launcher checks that 64 * k * 2 stays well below 2^32)
+      const bool inside = k_base + 8 * piece_lane < k_rows;
+      const uint32_t first = token_load_base + (uint32_t)k_base * 2u;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = buffer_load16(b_buffer, inside ? first + i * token_load_step : 0xFFFFFF00u, 0);
+      return;
+    }
     if (MODE == kSkinnyBFull && b_fits && k_base + IMG_ROWS <= k_rows) {
       // the whole image lies inside B (wave-uniform test): 8 KiB of consecutive memory, no per-piece checks
       const uint32_t image = (uint32_t)k_base * (NC * 2);
@@ -873,6 +1051,14 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
       }
       return;
     }
+    if (TOKENS) {
+      // token = token_lane + TPI i with token_lane < TPI (a power of two): the two terms share no bits, so the swizzle of
+      // piece i differs from that of piece 0 by a compile-time XOR
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        *reinterpret_cast<u32x4_t*>(region + (token_store_base ^ (uint32_t)(token_swizzle<TOKEN_ROW_BYTES>(TPI * i) << 4)) + i * 1024) = v[i];
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4_t*>(region + (lane + i * 64) * 16) = v[i];
   };
@@ -890,8 +1076,20 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   const int chunk8 = (NC >= 32 ? ((lane & 31) >> 4) * 4 : 0) + (i16 & 3);  // 8-byte piece of the 32-column fragment
   const char* lane_ptr = region + (8 * gb + (i16 >> 2)) * ROW_BYTES + chunk8 * 8;
 
+  // token-major image: this lane's token row and swizzle; K step s of the image needs pieces 4 s + gb and 4 s + 2 + gb
+  const int token_col = NC >= 32 ? (lane & 31) : i16;
+  const uint32_t token_read_base = (uint32_t)token_col * TOKEN_ROW_BYTES + (uint32_t)((gb ^ token_swizzle<TOKEN_ROW_BYTES>(token_col)) << 4);
   auto frag = [&](int image_step, int f) __attribute__((always_inline)) {
     u32x8_t raw;
+    if (TOKENS) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const u32x4_t t = *reinterpret_cast<const u32x4_t*>(
+            region + (token_read_base ^ (uint32_t)((4 * image_step + 2 * h) << 4)) + f * 32 * TOKEN_ROW_BYTES);
+        raw[4 * h] = t.x; raw[4 * h + 1] = t.y; raw[4 * h + 2] = t.z; raw[4 * h + 3] = t.w;
+      }
+      return __builtin_bit_cast(half16_t, raw);
+    }
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int row_const = image_step * 32 + 4 * (q & 1) + 16 * (q >> 1);
@@ -1010,6 +1208,7 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
 
   smfmac_drain();
   // ---- add the NW partial tiles through LDS: region of wavefront w := its R tiles as [r][32 rows][NC cols] fp32
+  constexpr int GROUP_ROWS = R * kRowBlock;
   {
     float* tile = reinterpret_cast<float*>(region);
     const int col = lane & 31;
@@ -1021,11 +1220,32 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
             const int row = 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-            tile[(r * 32 + row) * NC + f * 32 + col] = acc[r][f][v];
+            // token-major: [token][weight row of the group], the row index XOR-swizzled by the token so that neither
+            // these stores (32 tokens, one row) nor the reads below (one token, consecutive rows) collide in a bank
+            if (TOKENS) tile[(f * 32 + col) * GROUP_ROWS + ((r * 32 + row) ^ col)] = acc[r][f][v];
+            else tile[(r * 32 + row) * NC + f * 32 + col] = acc[r][f][v];
           }
     }
   }
   __syncthreads();
+  if (TOKENS) {
+    for (int idx = tid; idx < GROUP_ROWS * NC; idx += NT) {
+      const int local = idx % GROUP_ROWS, token = idx / GROUP_ROWS;
+      const int pos = token * GROUP_ROWS + (local ^ (token & 31));
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) sum += reinterpret_cast<const float*>(bs + w * kSkinnyRegion)[pos];
+      const int row = rb_first * kRowBlock + local;
+      if (token < p.n && row < p.m) {
+        if (p.bias) sum += p.bias_f16 ? (float)reinterpret_cast<const _Float16*>(p.bias)[row]
+                                      : reinterpret_cast<const float*>(p.bias)[row];
+        const size_t o = (size_t)token * p.m + row;
+        if (p.d_f16) reinterpret_cast<_Float16*>(p.d)[o] = (_Float16)sum;
+        else reinterpret_cast<float*>(p.d)[o] = sum;
+      }
+    }
+    return;
+  }
   for (int idx = tid; idx < R * kRowBlock * NC; idx += NT) {
     float sum = 0.f;
 #pragma unroll
@@ -1066,12 +1286,14 @@ __global__ __launch_bounds__(256) void pad_b_kernel(const _Float16* __restrict__
 // =====================================================================================================
 // splitk_reduce_kernel: d = alpha * (sum over splits, in split order, of the fp32 partial sums) + beta * c.
 // Elementwise over the m * n results; VEC = 4 when the element count and the alignment of c and d allow it.
+// Linear-layer form: bias (row_length values, may be null) is added instead, element i taking bias[i % row_length].
 // =====================================================================================================
 template <int VEC>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, int splits, size_t stride,
                                                             const void* __restrict__ c, void* __restrict__ d,
                                                             size_t total, float alpha, float beta, int c_f16,
-                                                            int d_f16) {
+                                                            int d_f16, const void* __restrict__ bias, int bias_f16,
+                                                            int row_length) {
   const size_t first = ((size_t)blockIdx.x * 256 + threadIdx.x) * VEC;
   if (first >= total) return;
   float x[VEC];
@@ -1095,9 +1317,14 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
       x[j] = x[j] + beta * cv;
     }
   }
+  if (bias) {
+    const size_t at = first % (size_t)row_length;  // row_length is a multiple of 4: a vector never wraps
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+      x[j] += bias_f16 ? (float)reinterpret_cast<const _Float16*>(bias)[at + j] : reinterpret_cast<const float*>(bias)[at + j];
+  }
   if (VEC == 4) {
     if (d_f16) {
-      typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
       *reinterpret_cast<half4_t*>(reinterpret_cast<_Float16*>(d) + first) =
           half4_t{(_Float16)x[0], (_Float16)x[1 % VEC], (_Float16)x[2 % VEC], (_Float16)x[3 % VEC]};
     } else {
@@ -1127,13 +1354,13 @@ hipError_t launch_pack(const void* w, void* a, void* e, int m, int k, int prune,
   return hipGetLastError();
 }
 
-template <int WM, int WN, int FM, int FN, bool DMA>
+template <int WM, int WN, int FM, int FN, bool DMA, bool TOKENS = false>
 static hipError_t launch_gemm_cfg(GemmArgs args, hipStream_t stream) {
   using TS = TileShape<WM, WN, FM, FN>;
   args.tiles_m = (args.m + TS::BM - 1) / TS::BM;
   args.tiles_n = (args.n + TS::BN - 1) / TS::BN;
   const int lds = DMA ? TS::LDS_BYTES : TS::STAGE_BYTES;
-  auto kern = gemm_kernel<WM, WN, FM, FN, DMA>;
+  auto kern = gemm_kernel<WM, WN, FM, FN, DMA, TOKENS>;
   // the dynamic-LDS limit is a per-device attribute of the kernel; threads that race here set the same value
   static std::atomic<bool> attr_done[64] = {};
   int device = 0;
@@ -1173,6 +1400,54 @@ static hipError_t launch_gemm_pass(GemmArgs args, int tile_config, hipStream_t s
   }
 }
 
+hipError_t launch_gemm_tokens(GemmArgs args, int tile_config, hipStream_t stream) {
+  if (prepared_bytes(args.m, args.k) >= (size_t(1) << 32)) return hipErrorInvalidValue;  // 32-bit copy offsets
+  if ((reinterpret_cast<uintptr_t>(args.b) & 15) != 0 || (size_t)args.k * 256 * 2 >= (size_t(1) << 32))
+    return hipErrorInvalidValue;  // 16-byte copies of x; 32-bit offsets inside a tile's token rows
+  const int chunks = (args.k + kChunkK - 1) / kChunkK;
+  args.ldb = args.k;
+  args.alpha = 1.f;
+  args.beta = 0.f;
+  args.c = nullptr;
+  auto pass = [&](GemmArgs a) {
+    a.vector_epilogue = (reinterpret_cast<uintptr_t>(a.d) & 15) == 0 && a.m % 8 == 0 &&
+                        (reinterpret_cast<uintptr_t>(a.bias) & 15) == 0;
+    switch (tile_config) {
+      case kTile256x128w: return launch_gemm_cfg<2, 2, 4, 2, true, true>(a, stream);
+      case kTile128x128s: return launch_gemm_cfg<2, 2, 2, 2, true, true>(a, stream);
+      case kTile512x128w8: return launch_gemm_cfg<4, 2, 4, 2, true, true>(a, stream);
+      case kTile256x128w8: return launch_gemm_cfg<4, 2, 2, 2, true, true>(a, stream);
+      case kTile128x128w8: return launch_gemm_cfg<2, 4, 2, 1, true, true>(a, stream);
+      case kTile64x128: return launch_gemm_cfg<2, 2, 1, 2, true, true>(a, stream);
+      default: return hipErrorInvalidValue;  // the tiles the automatic choice uses
+    }
+  };
+  if (args.splits <= 1) {
+    args.splits = 1;
+    args.chunks_per_split = chunks;
+    return pass(args);
+  }
+  if (args.chunks_per_split < 1 || (long)(args.splits - 1) * args.chunks_per_split >= chunks || !args.split_ws)
+    return hipErrorInvalidValue;  // an empty split would address past the prepared operand
+  // pass 1: raw fp32 partial sums per split, token-major like y; pass 2: ordered sum and bias
+  GemmArgs first = args;
+  first.d = args.split_ws;
+  first.d_f16 = 0;
+  first.bias = nullptr;
+  if (hipError_t st = pass(first); st != hipSuccess) return st;
+  const size_t total = (size_t)args.m * args.n;
+  const bool vec = (reinterpret_cast<uintptr_t>(args.d) & 15) == 0;  // m is a multiple of 64
+  if (vec)
+    hipLaunchKernelGGL(splitk_reduce_kernel<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream,
+                       args.split_ws, args.splits, total, nullptr, args.d, total, 1.f, 0.f, 0, args.d_f16, args.bias,
+                       args.bias_f16, args.m);
+  else
+    hipLaunchKernelGGL(splitk_reduce_kernel<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                       args.split_ws, args.splits, total, nullptr, args.d, total, 1.f, 0.f, 0, args.d_f16, args.bias,
+                       args.bias_f16, args.m);
+  return hipGetLastError();
+}
+
 hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
   if (prepared_bytes(args.m, args.k) >= (size_t(1) << 32)) return hipErrorInvalidValue;  // 32-bit copy offsets
   args.ldb = args.n;
@@ -1208,11 +1483,11 @@ hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
   if (vec)
     hipLaunchKernelGGL(splitk_reduce_kernel<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream,
                        args.split_ws, args.splits, total, args.c, args.d, total, args.alpha, args.beta, args.c_f16,
-                       args.d_f16);
+                       args.d_f16, nullptr, 0, 1);
   else
     hipLaunchKernelGGL(splitk_reduce_kernel<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
                        args.split_ws, args.splits, total, args.c, args.d, total, args.alpha, args.beta, args.c_f16,
-                       args.d_f16);
+                       args.d_f16, nullptr, 0, 1);
   return hipGetLastError();
 }
 
@@ -1241,6 +1516,25 @@ static hipError_t launch_skinny_cfg(const SkinnyArgs& args, hipStream_t stream) 
   if (args.n == 8 && (address & 15) == 0) return launch_skinny_mode<NW, R, kSkinnyB8, 16>(args, stream);
   if (args.n == 4 && (address & 7) == 0) return launch_skinny_mode<NW, R, kSkinnyB4, 16>(args, stream);
   return launch_skinny_mode<NW, R, kSkinnyBScalar, 16>(args, stream);
+}
+
+template <int NW, int R>
+static hipError_t launch_skinny_tokens_cfg(const SkinnyArgs& args, hipStream_t stream) {
+  if (args.n > 32) return launch_skinny_mode<NW, 1, kSkinnyBTokens, 64>(args, stream);
+  if (args.n > 16) return launch_skinny_mode<NW, (R > 2 ? 2 : R), kSkinnyBTokens, 32>(args, stream);
+  return launch_skinny_mode<NW, R, kSkinnyBTokens, 16>(args, stream);
+}
+
+hipError_t launch_skinny_tokens(SkinnyArgs args, int rows_per_group, hipStream_t stream) {
+  if (args.n < 1 || args.n > kSkinnyMaxN) return hipErrorInvalidValue;
+  // 16-byte loads of x; lane offsets of up to 64 token rows must stay below the "outside" offset of the kernel
+  if ((reinterpret_cast<uintptr_t>(args.b) & 15) != 0 || (size_t)args.k * 64 * 2 >= 0xFFFFFF00u) return hipErrorInvalidValue;
+  switch (rows_per_group) {
+    case 32: return launch_skinny_tokens_cfg<16, 1>(args, stream);
+    case 64: return launch_skinny_tokens_cfg<8, 2>(args, stream);
+    case 128: return launch_skinny_tokens_cfg<8, 4>(args, stream);
+    default: return hipErrorInvalidValue;
+  }
 }
 
 hipError_t launch_skinny(SkinnyArgs args, int rows_per_group, hipStream_t stream) {

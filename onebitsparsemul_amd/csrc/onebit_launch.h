@@ -28,6 +28,9 @@ struct GemmArgs {
   // take the slower element-copy variant. ldb (elements between B rows) is filled by the launcher.
   _Float16* b_pad;
   int ldb;
+  // linear-layer form (launch_gemm_tokens) only: m values added to every token's row of y, may be null
+  const void* bias;
+  int bias_f16;
 };
 
 struct SkinnyArgs {
@@ -39,12 +42,20 @@ struct SkinnyArgs {
   int kc_total;
   float alpha, beta;
   int c_f16, d_f16;
+  // token-major form (launch_skinny_tokens) only: b is x (n tokens x k), d is y (n tokens x m), alpha, beta and c are
+  // not used, bias (m values, may be null) is added to every token's row
+  const void* bias;
+  int bias_f16;
 };
 
 enum TileConfig { kTile512x128 = 0, kTile256x128 = 1, kTile128x128 = 2, kTile256x256 = 3, kTile256x128w = 4, kTile512x128t = 5, kTile128x128s = 6, kTile256x64 = 7, kTile256x256w8 = 8, kTile512x128w8 = 9, kTile256x128w8 = 10, kTile128x128w8 = 11, kTile64x128 = 12, kTileAuto = -1 };
 
 hipError_t launch_prepare(const void* a, const void* e, void* prep, int m, int k, int layout, hipStream_t stream);
 hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream);
+// The linear layer's form of the main kernel: b is x (n tokens x k, token-major, 16-byte aligned), d is y (n tokens x
+// m), y = x W^T + bias; c, alpha, beta and the padded copy of B are not used, splits / chunks_per_split / split_ws as in
+// launch_gemm. Tiles 4, 6, 9, 10, 11, 12.
+hipError_t launch_gemm_tokens(GemmArgs args, int tile_config, hipStream_t stream);
 // dense fp16 (m x k) -> one-bit values `a` and metadata `e`; prune != 0 applies the 2:4 magnitude mask first
 hipError_t launch_pack(const void* w, void* a, void* e, int m, int k, int prune, int layout, hipStream_t stream);
 
@@ -52,5 +63,8 @@ hipError_t launch_pack(const void* w, void* a, void* e, int m, int k, int prune,
 // most 64; n > 32: always 32).
 constexpr int kSkinnyMaxN = 64;
 hipError_t launch_skinny(SkinnyArgs args, int rows_per_group, hipStream_t stream);
+// The linear layer's form of the same kernel: y[t][r] = sum_k W[r][k] x[t][k] + bias[r] for n <= 64 tokens, x and y
+// token-major (x 16-byte aligned).
+hipError_t launch_skinny_tokens(SkinnyArgs args, int rows_per_group, hipStream_t stream);
 
 }  // namespace onebit

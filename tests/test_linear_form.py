@@ -1,0 +1,149 @@
+"""Linear-layer form of the prepared product (token-major x and y, fused bias) against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from onebitsparsemul_amd import _native, synthetic
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _defaults():
+    _native.set_tile_config(-1)
+    _native.set_skinny_enabled(True)
+    _native.set_skinny_rows(-1)
+    _native.set_split_k(-1)
+    yield
+    _native.set_tile_config(-1)
+    _native.set_skinny_enabled(True)
+    _native.set_skinny_rows(-1)
+    _native.set_split_k(-1)
+
+
+def _expected(dense, x, bias, y_dtype):
+    """y = (W x^T)^T + bias with the oracle's host GEMM (fp32 accumulation; exact for small integers)."""
+    d = oracle.host_gemm(dense, np.ascontiguousarray(x.T), d_dtype=oracle.F32, acc="f32").T
+    if bias is not None:
+        d = d + bias.astype(np.float32)[None, :]
+    return d.astype(y_dtype)
+
+
+@pytest.mark.parametrize("rows", [-1, 32, 64, 128])
+@pytest.mark.parametrize("tokens", [1, 5, 16, 17, 32, 33, 64])
+@pytest.mark.parametrize("m,k", [(256, 512), (192, 1056), (1024, 4096), (448, 8480)])
+def test_linear_form_small_token_counts(rows, tokens, m, k):
+    _native.set_skinny_rows(rows)
+    a, meta = synthetic.make_weight(m, k, seed=m + k + tokens)
+    dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
+    x = synthetic.make_b(tokens, k, seed=tokens, kind="int")           # (tokens, k) small integers
+    bias = synthetic.make_b(1, m, seed=tokens + 1, kind="int").reshape(m)
+    prep = _native.prepare(a.cuda(), meta.cuda(), m, k)
+    for y_dtype, b in ((torch.float32, bias), (torch.float16, None), (torch.float16, bias.float())):
+        y = torch.full((tokens, m), float("nan"), dtype=y_dtype, device="cuda")
+        _native.linear_prepared(prep, x.cuda(), y, m, k, bias=b.cuda() if b is not None else None)
+        torch.cuda.synchronize()
+        want = _expected(dense, x.numpy().astype(np.float32), b.numpy() if b is not None else None,
+                         np.float32 if y_dtype == torch.float32 else np.float16)
+        assert np.array_equal(y.cpu().numpy(), want), (y_dtype, b is not None)
+
+
+@pytest.mark.parametrize("tile", [-1, 4, 6, 9, 10, 11, 12])
+@pytest.mark.parametrize("tokens,m,k", [(65, 256, 512), (128, 192, 1056), (200, 1024, 2048), (1000, 640, 544), (16, 256, 800),
+                                        (520, 4096, 512)])
+def test_linear_form_main_kernel(tile, tokens, m, k):
+    _native.set_tile_config(tile)
+    _native.set_skinny_enabled(False)
+    a, meta = synthetic.make_weight(m, k, seed=m + k + tokens)
+    dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
+    x = synthetic.make_b(tokens, k, seed=tokens, kind="int")
+    bias = synthetic.make_b(1, m, seed=tokens + 1, kind="int").reshape(m)
+    prep = _native.prepare(a.cuda(), meta.cuda(), m, k)
+    for y_dtype, b in ((torch.float32, bias), (torch.float16, None), (torch.float16, bias.float())):
+        y = torch.full((tokens, m), float("nan"), dtype=y_dtype, device="cuda")
+        _native.linear_prepared(prep, x.cuda(), y, m, k, bias=b.cuda() if b is not None else None)
+        torch.cuda.synchronize()
+        want = _expected(dense, x.numpy().astype(np.float32), b.numpy() if b is not None else None,
+                         np.float32 if y_dtype == torch.float32 else np.float16)
+        assert np.array_equal(y.cpu().numpy(), want), (y_dtype, b is not None)
+
+
+@pytest.mark.parametrize("splits", [-1, 2, 3, 16])
+@pytest.mark.parametrize("tokens,m,k", [(128, 256, 4096), (72, 192, 2080), (264, 1024, 1024)])
+def test_linear_form_k_split_over_workgroups(splits, tokens, m, k):
+    _native.set_split_k(splits)
+    _native.set_skinny_enabled(False)
+    a, meta = synthetic.make_weight(m, k, seed=splits + m + k)
+    dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
+    x = synthetic.make_b(tokens, k, seed=tokens, kind="int")
+    bias = synthetic.make_b(1, m, seed=tokens + 1, kind="int").reshape(m)
+    prep = _native.prepare(a.cuda(), meta.cuda(), m, k)
+    for y_dtype, b in ((torch.float32, bias), (torch.float16, None), (torch.float16, bias.float())):
+        y = torch.full((tokens, m), float("nan"), dtype=y_dtype, device="cuda")
+        _native.linear_prepared(prep, x.cuda(), y, m, k, bias=b.cuda() if b is not None else None)
+        torch.cuda.synchronize()
+        want = _expected(dense, x.numpy().astype(np.float32), b.numpy() if b is not None else None,
+                         np.float32 if y_dtype == torch.float32 else np.float16)
+        assert np.array_equal(y.cpu().numpy(), want), (y_dtype, b is not None)
+    # result 2 bytes past a 16-byte boundary: the element form of the reduction
+    store = torch.full((tokens * m + 1,), float("nan"), dtype=torch.float16, device="cuda")
+    y = store[1:].view(tokens, m)
+    _native.linear_prepared(prep, x.cuda(), y, m, k, bias=bias.cuda())
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), _expected(dense, x.numpy().astype(np.float32), bias.numpy(), np.float16))
+
+
+@pytest.mark.parametrize("tokens", [8, 300])
+def test_linear_form_result_not_16_byte_aligned(tokens):
+    m, k = 320, 1024
+    a, meta = synthetic.make_weight(m, k, seed=3)
+    dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
+    x = synthetic.make_b(tokens, k, seed=4, kind="int")
+    prep = _native.prepare(a.cuda(), meta.cuda(), m, k)
+    store = torch.full((tokens * m + 1,), float("nan"), dtype=torch.float16, device="cuda")
+    y = store[1:].view(tokens, m)  # 2 bytes past a 16-byte boundary
+    _native.linear_prepared(prep, x.cuda(), y, m, k)
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), _expected(dense, x.numpy().astype(np.float32), None, np.float16))
+    # aligned result, bias 2 bytes past a 16-byte boundary
+    bias = synthetic.make_b(1, m + 1, seed=5, kind="int").reshape(m + 1).cuda()[1:]
+    y2 = torch.full((tokens, m), float("nan"), dtype=torch.float16, device="cuda")
+    _native.linear_prepared(prep, x.cuda(), y2, m, k, bias=bias)
+    torch.cuda.synchronize()
+    assert np.array_equal(y2.cpu().numpy(), _expected(dense, x.numpy().astype(np.float32), bias.cpu().numpy(), np.float16))
+
+
+def test_linear_form_rejects_misaligned_x():
+    m, k, tokens = 64, 256, 4
+    a, meta = synthetic.make_weight(m, k, seed=3)
+    prep = _native.prepare(a.cuda(), meta.cuda(), m, k)
+    store = torch.zeros(tokens * k + 1, dtype=torch.float16, device="cuda")
+    y = torch.empty((tokens, m), dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError, match="16-byte aligned"):
+        _native.linear_prepared(prep, store[1:].view(tokens, k), y, m, k)
+
+
+@pytest.mark.parametrize("lead", [(7,), (3, 70), (2, 2, 9)])
+@pytest.mark.parametrize("x_dtype", [torch.float16, torch.float32])
+def test_layer_forward_with_bias(lead, x_dtype):
+    """BinaryLinear_2_4.forward goes through the linear form: any leading shape, fp16 or fp32 activations, bias fused"""
+    import onebitsparsemul_amd as ob
+    out_f, in_f = 640, 512
+    torch.manual_seed(0)
+    layer = ob.BinaryLinear_2_4(in_f, out_f)
+    layer.pack(torch.randn(out_f, in_f).half())
+    layer.bias = torch.randint(-3, 4, (out_f,)).to(torch.float16)
+    x = torch.randint(-4, 5, lead + (in_f,)).to(x_dtype)
+    want = ob.py_binary_gemm(x.reshape(-1, in_f).float(), layer.packed_binary_sparse, layer.meta) + layer.bias.float()
+    layer = layer.cuda()
+    layer.bias = layer.bias.cuda()
+    got = layer(x.cuda())
+    torch.cuda.synchronize()
+    assert got.dtype == x_dtype and tuple(got.shape) == lead + (out_f,)
+    assert torch.equal(got.cpu().float().reshape(-1, out_f), want)
+    # a view that does not start on a 16-byte boundary
+    store = torch.zeros(x.numel() + 1, dtype=torch.float16, device="cuda")
+    store[1:] = x.reshape(-1).cuda().half()
+    got2 = layer(store[1:].view(*lead, in_f))
+    assert torch.equal(got2.cpu().float().reshape(-1, out_f), want)
