@@ -99,7 +99,7 @@ int onebit_sparse_pack(const void *weight, int m, int k, int prune, void *a, voi
 const char *onebit_sparse_last_error(void);
 
 /* Tuning / test hooks: force a tile configuration of the main kernel (-1 = automatic) and choose whether
- * shapes with n <= 32 (n <= 64 when m <= 16384) use the split-K kernel (1, default) or the main kernel (0).
+ * shapes with n <= 32 (n <= 64 when m <= 40960) use the split-K kernel (1, default) or the main kernel (0).
  * Tile codes 0-11 are the TileConfig values of csrc/onebit_launch.h. Process-wide. */
 void onebit_sparse_set_tile_config(int tile_config);
 void onebit_sparse_set_skinny_enabled(int enabled);

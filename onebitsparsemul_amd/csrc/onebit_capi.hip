@@ -183,14 +183,16 @@ struct LaunchPlan {
 
 LaunchPlan choose_launch(int m, int n, int k, bool b_16_byte_aligned) {
   LaunchPlan plan{};
-  // 32 < n <= 64: every 32-row workgroup of the split-K kernel stages all of B, which the main kernel's tiles
-  // overtake from about 16k rows on (28672 x 64 x 8192: 43 us against 58 us; 11008 x 64 x 4096: 21 against 17)
-  const bool skinny_shape = n <= 32 || (n <= onebit::kSkinnyMaxN && m <= 16384);
+  // 32 < n <= 64: every 64-row workgroup of the split-K kernel stages all of B, which the main kernel's tiles overtake
+  // from about 48k rows on (n = 64: 28672 x 8192 32 us against 42; 32768 x 4096 20 against 26; 49152 x 4096 32.5
+  // against 34.4; 65536 x 8192 66 against 68, at n = 40 77 against 66; 131072 x 2048 51 against 35)
+  const bool skinny_shape = n <= 32 || (n <= onebit::kSkinnyMaxN && m <= 40960);
   if (skinny_shape && g_skinny_enabled.load()) {
     int rows = g_skinny_rows.load();
     // the largest row group that still gives about two workgroups per three compute units (measured: larger groups
     // re-read B less often, but idle compute units cost more)
-    if (rows <= 0) rows = n > 32 ? 32 : (m / 128 >= 160 && n <= 16) ? 128 : (m / 64 >= 160) ? 64 : 32;
+    // (n > 32: two column fragments per row block, at most two row blocks per wavefront)
+    if (rows <= 0) rows = (m / 128 >= 160 && n <= 32) ? 128 : (m / 64 >= 160) ? 64 : 32;
     plan.split_k_kernel = 1;
     plan.rows_or_tile = rows;
     plan.splits = 1;

@@ -885,7 +885,8 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
 // fp32 partial tile per row block. The prepared operand and the next image are loaded into registers while the
 // current one is multiplied. Wavefronts never wait for one another inside the K loop (LDS operations of one
 // wavefront execute in order). The NW partial tiles of a row block are added through LDS in wavefront order
-// (deterministic) and the epilogue is applied. grid = M / (32 R) workgroups; no global workspace, no atomics.
+// (deterministic; the tiles take the place of the images, as many row blocks per round as fit the 8 KiB) and the
+// epilogue is applied. grid = M / (32 R) workgroups; no global workspace, no atomics.
 // =====================================================================================================
 #ifndef ONEBIT_EXP_SKINNY
 #define ONEBIT_EXP_SKINNY 0  // measurement builds (results wrong): 1 no B reloads, 2 one fragment group per chunk, 3 one expansion per chunk, 4 loads and image stores only
@@ -940,7 +941,9 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   constexpr int TILE_BYTES = kRowBlock * NC * 4;       // one fp32 partial tile
   static_assert(NC == 16 || NC == 32 || NC == 64, "image width");
   static_assert(MODE != kSkinnyB4 || NC == 16, "the 8-byte-row mode is for 16 columns");
-  static_assert(R * TILE_BYTES <= kSkinnyRegion, "partial tiles reuse the wavefront's image memory");
+  // the partial tiles reuse the wavefront's image memory, RT row blocks per round of the final reduction
+  constexpr int RT = R * TILE_BYTES <= kSkinnyRegion ? R : kSkinnyRegion / TILE_BYTES;
+  static_assert(RT >= 1 && R % RT == 0, "the row blocks must divide into whole reduction rounds");
   constexpr bool TOKENS = MODE == kSkinnyBTokens;
   constexpr int PPT = IMG_ROWS / 8;                    // token-major image: 16-byte pieces per token row
   constexpr int TPI = 64 / PPT;                        // ... and tokens covered by the 64 pieces of one wavefront load
@@ -1208,59 +1211,65 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
 
   smfmac_drain();
   // ---- add the NW partial tiles through LDS: region of wavefront w := its R tiles as [r][32 rows][NC cols] fp32
-  constexpr int GROUP_ROWS = R * kRowBlock;
-  {
-    float* tile = reinterpret_cast<float*>(region);
-    const int col = lane & 31;
-    if (col < NC) {
+  constexpr int ROUND_ROWS = RT * kRowBlock;
 #pragma unroll
-      for (int r = 0; r < R; ++r)
+  for (int round = 0; round < R / RT; ++round) {
+    if (round > 0) __syncthreads();  // the previous round's tiles have been read
+    {
+      float* tile = reinterpret_cast<float*>(region);
+      const int col = lane & 31;
+      if (col < NC) {
 #pragma unroll
-        for (int f = 0; f < NF; ++f)
+        for (int rr = 0; rr < RT; ++rr)
 #pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const int row = 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-            // token-major: [token][weight row of the group], the row index XOR-swizzled by the token so that neither
-            // these stores (32 tokens, one row) nor the reads below (one token, consecutive rows) collide in a bank
-            if (TOKENS) tile[(f * 32 + col) * GROUP_ROWS + ((r * 32 + row) ^ col)] = acc[r][f][v];
-            else tile[(r * 32 + row) * NC + f * 32 + col] = acc[r][f][v];
+          for (int f = 0; f < NF; ++f)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              const int row = 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+              const float value = acc[round * RT + rr][f][v];
+              // token-major: [token][weight row of the round], the row index XOR-swizzled by the token so that neither
+              // these stores (32 tokens, one row) nor the reads below (one token, consecutive rows) collide in a bank
+              if (TOKENS) tile[(f * 32 + col) * ROUND_ROWS + ((rr * 32 + row) ^ col)] = value;
+              else tile[(rr * 32 + row) * NC + f * 32 + col] = value;
+            }
+      }
+    }
+    __syncthreads();
+    const int round_row0 = rb_first * kRowBlock + round * ROUND_ROWS;
+    if (TOKENS) {
+      for (int idx = tid; idx < ROUND_ROWS * NC; idx += NT) {
+        const int local = idx % ROUND_ROWS, token = idx / ROUND_ROWS;
+        const int pos = token * ROUND_ROWS + (local ^ (token & 31));
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) sum += reinterpret_cast<const float*>(bs + w * kSkinnyRegion)[pos];
+        const int row = round_row0 + local;
+        if (token < p.n && row < p.m) {
+          if (p.bias) sum += p.bias_f16 ? (float)reinterpret_cast<const _Float16*>(p.bias)[row]
+                                        : reinterpret_cast<const float*>(p.bias)[row];
+          const size_t o = (size_t)token * p.m + row;
+          if (p.d_f16) reinterpret_cast<_Float16*>(p.d)[o] = (_Float16)sum;
+          else reinterpret_cast<float*>(p.d)[o] = sum;
+        }
+      }
+    } else {
+      for (int idx = tid; idx < ROUND_ROWS * NC; idx += NT) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) sum += reinterpret_cast<const float*>(bs + w * kSkinnyRegion)[idx];
+        const int col = idx % NC;
+        const int row = round_row0 + idx / NC;
+        if (col < p.n && row < p.m) {
+          const size_t o = (size_t)row * p.n + col;
+          float x = p.alpha * sum;
+          if (p.beta != 0.f) {
+            const float cv = p.c_f16 ? (float)reinterpret_cast<const _Float16*>(p.c)[o] : reinterpret_cast<const float*>(p.c)[o];
+            x = x + p.beta * cv;
           }
-    }
-  }
-  __syncthreads();
-  if (TOKENS) {
-    for (int idx = tid; idx < GROUP_ROWS * NC; idx += NT) {
-      const int local = idx % GROUP_ROWS, token = idx / GROUP_ROWS;
-      const int pos = token * GROUP_ROWS + (local ^ (token & 31));
-      float sum = 0.f;
-#pragma unroll
-      for (int w = 0; w < NW; ++w) sum += reinterpret_cast<const float*>(bs + w * kSkinnyRegion)[pos];
-      const int row = rb_first * kRowBlock + local;
-      if (token < p.n && row < p.m) {
-        if (p.bias) sum += p.bias_f16 ? (float)reinterpret_cast<const _Float16*>(p.bias)[row]
-                                      : reinterpret_cast<const float*>(p.bias)[row];
-        const size_t o = (size_t)token * p.m + row;
-        if (p.d_f16) reinterpret_cast<_Float16*>(p.d)[o] = (_Float16)sum;
-        else reinterpret_cast<float*>(p.d)[o] = sum;
+          if (p.d_f16) reinterpret_cast<_Float16*>(p.d)[o] = (_Float16)x;
+          else reinterpret_cast<float*>(p.d)[o] = x;
+        }
       }
-    }
-    return;
-  }
-  for (int idx = tid; idx < R * kRowBlock * NC; idx += NT) {
-    float sum = 0.f;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) sum += reinterpret_cast<const float*>(bs + w * kSkinnyRegion)[idx];
-    const int col = idx % NC;
-    const int row = rb_first * kRowBlock + idx / NC;
-    if (col < p.n && row < p.m) {
-      const size_t o = (size_t)row * p.n + col;
-      float x = p.alpha * sum;
-      if (p.beta != 0.f) {
-        const float cv = p.c_f16 ? (float)reinterpret_cast<const _Float16*>(p.c)[o] : reinterpret_cast<const float*>(p.c)[o];
-        x = x + p.beta * cv;
-      }
-      if (p.d_f16) reinterpret_cast<_Float16*>(p.d)[o] = (_Float16)x;
-      else reinterpret_cast<float*>(p.d)[o] = x;
     }
   }
 }
@@ -1501,13 +1510,14 @@ static hipError_t launch_skinny_mode(const SkinnyArgs& args, hipStream_t stream)
 template <int NW, int R>
 static hipError_t launch_skinny_cfg(const SkinnyArgs& args, hipStream_t stream) {
   const uintptr_t address = reinterpret_cast<uintptr_t>(args.b);
-  if (args.n > 32) {  // 64-column images; one partial tile fills the image memory
-    if (args.n == 64 && (address & 15) == 0) return launch_skinny_mode<NW, 1, kSkinnyBFull, 64>(args, stream);
-    if (args.n % 8 == 0 && (address & 15) == 0) return launch_skinny_mode<NW, 1, kSkinnyB8, 64>(args, stream);
-    return launch_skinny_mode<NW, 1, kSkinnyBScalar, 64>(args, stream);
+  if (args.n > 32) {  // 64-column images, two column fragments: at most two row blocks fit the registers
+    constexpr int R64 = R > 2 ? 2 : R;
+    if (args.n == 64 && (address & 15) == 0) return launch_skinny_mode<NW, R64, kSkinnyBFull, 64>(args, stream);
+    if (args.n % 8 == 0 && (address & 15) == 0) return launch_skinny_mode<NW, R64, kSkinnyB8, 64>(args, stream);
+    return launch_skinny_mode<NW, R64, kSkinnyBScalar, 64>(args, stream);
   }
-  if (args.n > 16) {  // 32-column images; their two partial tiles per row block fill the image memory at R = 2
-    constexpr int R32 = R > 2 ? 2 : R;
+  if (args.n > 16) {  // 32-column images
+    constexpr int R32 = R;
     if (args.n == 32 && (address & 15) == 0) return launch_skinny_mode<NW, R32, kSkinnyBFull, 32>(args, stream);
     if (args.n % 8 == 0 && (address & 15) == 0) return launch_skinny_mode<NW, R32, kSkinnyB8, 32>(args, stream);
     return launch_skinny_mode<NW, R32, kSkinnyBScalar, 32>(args, stream);
@@ -1520,8 +1530,8 @@ static hipError_t launch_skinny_cfg(const SkinnyArgs& args, hipStream_t stream) 
 
 template <int NW, int R>
 static hipError_t launch_skinny_tokens_cfg(const SkinnyArgs& args, hipStream_t stream) {
-  if (args.n > 32) return launch_skinny_mode<NW, 1, kSkinnyBTokens, 64>(args, stream);
-  if (args.n > 16) return launch_skinny_mode<NW, (R > 2 ? 2 : R), kSkinnyBTokens, 32>(args, stream);
+  if (args.n > 32) return launch_skinny_mode<NW, (R > 2 ? 2 : R), kSkinnyBTokens, 64>(args, stream);
+  if (args.n > 16) return launch_skinny_mode<NW, R, kSkinnyBTokens, 32>(args, stream);
   return launch_skinny_mode<NW, R, kSkinnyBTokens, 16>(args, stream);
 }
 
@@ -1542,7 +1552,7 @@ hipError_t launch_skinny(SkinnyArgs args, int rows_per_group, hipStream_t stream
   switch (rows_per_group) {
     case 32: return launch_skinny_cfg<16, 1>(args, stream);  // sixteen wavefronts split K: small M
     case 64: return launch_skinny_cfg<8, 2>(args, stream);
-    case 128: return launch_skinny_cfg<8, 4>(args, stream);  // n > 16: 64-row groups
+    case 128: return launch_skinny_cfg<8, 4>(args, stream);  // n > 32: 64-row groups
     default: return hipErrorInvalidValue;
   }
 }

@@ -59,8 +59,7 @@ hipError_t launch_gemm_tokens(GemmArgs args, int tile_config, hipStream_t stream
 // dense fp16 (m x k) -> one-bit values `a` and metadata `e`; prune != 0 applies the 2:4 magnitude mask first
 hipError_t launch_pack(const void* w, void* a, void* e, int m, int k, int prune, int layout, hipStream_t stream);
 
-// Split-K kernel for n <= 64; rows_per_group (32, 64 or 128) = weight rows one workgroup covers (16 < n <= 32: at
-// most 64; n > 32: always 32).
+// Split-K kernel for n <= 64; rows_per_group (32, 64 or 128) = weight rows one workgroup covers (n > 32: at most 64).
 constexpr int kSkinnyMaxN = 64;
 hipError_t launch_skinny(SkinnyArgs args, int rows_per_group, hipStream_t stream);
 // The linear layer's form of the same kernel: y[t][r] = sum_k W[r][k] x[t][k] + bias[r] for n <= 64 tokens, x and y

@@ -139,9 +139,12 @@ def test_launch_plan_of_the_benchmark_shapes(_default_hooks):
         assert plan(11008, n, 4096) == dict(kernel="skinny_kernel", rows=64)
         assert plan(4096, n, 11008) == dict(kernel="skinny_kernel", rows=32)
     assert plan(28672, 16, 8192) == dict(kernel="skinny_kernel", rows=128)
-    assert plan(28672, 32, 8192) == dict(kernel="skinny_kernel", rows=64)
-    assert plan(11008, 64, 4096) == dict(kernel="skinny_kernel", rows=32)
-    assert plan(28672, 64, 8192)["kernel"] == "gemm_kernel"      # from 16k rows on the main kernel is faster
+    assert plan(28672, 32, 8192) == dict(kernel="skinny_kernel", rows=128)
+    assert plan(16384, 32, 4096) == dict(kernel="skinny_kernel", rows=64)
+    assert plan(4096, 64, 4096) == dict(kernel="skinny_kernel", rows=32)
+    assert plan(11008, 64, 4096) == dict(kernel="skinny_kernel", rows=64)   # 33 ... 64 columns: at most 64 rows
+    assert plan(28672, 64, 8192) == dict(kernel="skinny_kernel", rows=64)
+    assert plan(65536, 64, 8192)["kernel"] == "gemm_kernel"      # from about 48k rows on the main kernel is faster
     assert plan(4096, 65, 4096)["kernel"] == "gemm_kernel"
     # few tiles over a long K: split over workgroups; many tiles: never
     few = plan(4096, 128, 4096)

@@ -285,6 +285,23 @@ def test_one_call_entry_point_on_several_streams_keeps_the_reordered_weights_apa
         assert np.array_equal(o.cpu().numpy(), oracle.host_gemm(dense, b.numpy(), d_dtype=oracle.F32, acc="f32"))
 
 
+@pytest.mark.parametrize("m,k,n,rows", [(20480, 1024, 64, 64), (28672, 512, 40, 64), (28672, 1024, 32, 128), (20480, 768, 24, 128)])
+def test_split_k_kernel_large_m_row_groups(m, k, n, rows):
+    """the row groups the C ABI picks for many weight rows: 64 rows at 33 ... 64 columns, 128 rows at 17 ... 32
+    (partial tiles reduced in two rounds); exact on integers against the oracle"""
+    assert _native.describe_launch(m, n, k) == dict(kernel="skinny_kernel", rows=rows)
+    a, meta = synthetic.make_weight(m, k, seed=m + n)
+    dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
+    bi = synthetic.make_b(k, n, seed=n, kind="int")
+    exact = oracle.host_gemm(dense, bi.numpy(), d_dtype=oracle.F32, acc="f32")
+    assert np.array_equal(_run_prepared(a, meta, bi, m, n, k, out_dtype=torch.float32), exact)
+    prep = _native.prepare(a.cuda(), meta.cuda(), m, k)
+    y = torch.full((n, m), float("nan"), dtype=torch.float32, device="cuda")
+    _native.linear_prepared(prep, bi.T.contiguous().cuda(), y, m, k)
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), exact.T)
+
+
 def test_config3_split_k_is_deterministic_and_reusable():
     m, k, n = 4096, 11008, 16
     a, meta = synthetic.make_weight(m, k, seed=5)
