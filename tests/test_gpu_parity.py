@@ -581,6 +581,9 @@ def test_benchmark_cli_reference_check():
     assert benchmark.main(["--a_rows=512", "--n=256", "--a_cols=512", "--reference-check=true", "--iterations=2"]) == 0
     assert benchmark.main(["--a_rows=1024", "--n=16", "--a_cols=512", "--alpha=0.5", "--beta=1", "--reference-check=true",
                            "--iterations=2", "--fp16-out"]) == 0
+    # the linear layer's form: small and large token counts
+    assert benchmark.main(["--layer", "--a_rows=1024", "--n=16", "--a_cols=512", "--reference-check=true", "--iterations=2"]) == 0
+    assert benchmark.main(["--layer", "--a_rows=512", "--n=300", "--a_cols=512", "--reference-check=true", "--iterations=2"]) == 0
 
 
 def test_benchmark_cli_writes_json_and_csv(tmp_path):
