@@ -1,7 +1,11 @@
 // gfx950 kernels of the one-bit 2:4 sparse GEMM  D = alpha * A * B + beta * C.
 //   prepare_kernel  : reference operands (1-bit values, reordered 2-bit-index metadata) -> prepared operand
+//   pack_kernel     : dense fp16 weight -> the reference operands (2:4 magnitude mask, compression, one-bit values)
 //   gemm_kernel     : main SMFMAC kernel (B staged through LDS, A expanded in registers)
 //   skinny_kernel   : split-K kernel for N <= 64 (decode shapes)
+//   pad_b_kernel, splitk_reduce_kernel : helpers of the main kernel (unaligned B rows; K split over workgroups)
+// The two GEMM kernels also come in a token-major form for the linear layer, y = x W^T + bias with x and y stored
+// token by token (the transposes of B and D).
 // Replaces the CUTLASS specialisations of the reference (csrc/kernel.h:13-72, csrc/threadblock.h:62-233,
 // csrc/warp.h:18-690) with code written for 64-wide wavefronts; nothing is translated from them.
 #include "onebit_device.h"
@@ -881,7 +885,7 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
 // Workgroup = NW wavefronts that share R row blocks (32 rows each) and split K among themselves: wavefront w
 // takes the K chunks (of 256) w, w + NW, w + 2 NW, ... Each wavefront stages B rows in a private 8 KiB LDS region
 // as a zero-padded fp16 image of NC columns (NC = 16: the 256 rows of a chunk; NC = 32: 128 rows, two images per
-// chunk), feeds them to SMFMAC through transpose reads (one fragment serves the R row blocks) and keeps a 32x32
+// chunk; NC = 64: 64 rows, four images, two column fragments), feeds them to SMFMAC through transpose reads (one fragment serves the R row blocks) and keeps a 32x32
 // fp32 partial tile per row block. The prepared operand and the next image are loaded into registers while the
 // current one is multiplied. Wavefronts never wait for one another inside the K loop (LDS operations of one
 // wavefront execute in order). The NW partial tiles of a row block are added through LDS in wavefront order
