@@ -1,10 +1,12 @@
 """Swap the nn.Linear layers of a model for BinaryLinear_2_4 and account for the memory, as the reference's
 model script does for a TinyLlama checkpoint (tests/python/test_model_replace.py:22-56).
 
-    python -m onebitsparsemul_amd.replace [--model-dir DIR] [--device cuda]
+    python -m onebitsparsemul_amd.replace [--model-dir DIR] [--device cuda] [--time]
+    python -m onebitsparsemul_amd.replace --hidden 4096 --intermediate 11008 --layers 2 --time
 
 With --model-dir the Llama checkpoint in that local directory is loaded (nothing is downloaded); without it a
-small randomly initialised Llama of the same architecture is built, which exercises the same code path.
+small randomly initialised Llama of the same architecture is built (its sizes can be set), which exercises the same
+code path. --time also measures the forward pass over 16 and 512 tokens before and after the replacement.
 """
 import argparse
 
@@ -47,25 +49,51 @@ def replace_linear_layers(model, skip=()):
                 fp16_weight_gib=weight_params * 16 / 8 / gib, packed_weight_gib=weight_params * 1.5 / 8 / gib)
 
 
-def _build_model(model_dir, device):
+def _build_model(model_dir, device, hidden=512, intermediate=1408, layers=2):
     from transformers import LlamaConfig, LlamaForCausalLM
     if model_dir:
         model = LlamaForCausalLM.from_pretrained(model_dir, local_files_only=True)
     else:
-        config = LlamaConfig(vocab_size=4096, hidden_size=512, intermediate_size=1408, num_hidden_layers=2,
-                             num_attention_heads=8, num_key_value_heads=4, max_position_embeddings=256)
+        heads = max(1, hidden // 64)
+        config = LlamaConfig(vocab_size=4096, hidden_size=hidden, intermediate_size=intermediate,
+                             num_hidden_layers=layers, num_attention_heads=heads,
+                             num_key_value_heads=max(1, heads // 2), max_position_embeddings=1024)
         model = LlamaForCausalLM(config)
     return model.to(torch.float16).to(device)
+
+
+def _forward_ms(model, tokens, repeats=20):
+    """Average time of one forward pass over `tokens` (1 x T token ids), in milliseconds."""
+    with torch.no_grad():
+        for _ in range(3):
+            model(tokens)
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(repeats):
+            model(tokens)
+        stop.record()
+        torch.cuda.synchronize()
+    return start.elapsed_time(stop) / repeats
 
 
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--model-dir", default=None)
     ap.add_argument("--device", default="cuda")
+    ap.add_argument("--hidden", type=int, default=512, help="hidden size of the randomly initialised model")
+    ap.add_argument("--intermediate", type=int, default=1408)
+    ap.add_argument("--layers", type=int, default=2)
+    ap.add_argument("--time", action="store_true", help="time the forward pass before and after (GPU only)")
     args = ap.parse_args(argv)
-    model = _build_model(args.model_dir, args.device)
+    model = _build_model(args.model_dir, args.device, args.hidden, args.intermediate, args.layers)
     on_gpu = args.device.startswith("cuda")
     gib = 1024.0 ** 3
+    timed = {}
+    if on_gpu and args.time:
+        for count in (16, 512):
+            ids = torch.randint(0, model.config.vocab_size, (1, count), device=args.device)
+            timed[count] = [ids, _forward_ms(model, ids)]
     before = torch.cuda.memory_allocated(0) / gib if on_gpu else float("nan")
     stats = replace_linear_layers(model)
     if on_gpu:
@@ -84,6 +112,9 @@ def main(argv=None):
         with torch.no_grad():
             logits = model(tokens).logits
         print(f"forward through the replaced model: logits {tuple(logits.shape)}, finite={bool(torch.isfinite(logits).all())}")
+        for count, (ids, before_ms) in timed.items():
+            print(f"forward over {count} tokens: {before_ms:.3f} ms with nn.Linear (fp16), "
+                  f"{_forward_ms(model, ids):.3f} ms with BinaryLinear_2_4")
     return stats
 
 
