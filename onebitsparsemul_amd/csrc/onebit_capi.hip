@@ -120,7 +120,11 @@ int pick_tile(int m, int n) {
   const long mid = tiles(256, 128);
   if (mid >= 512) return onebit::kTile256x128w;
   if (mid >= 256) return onebit::kTile256x128w8;
-  if (tiles(128, 128) <= 256) return onebit::kTile128x128w8;
+  // at most one 128 x 128 workgroup per CU: eight wavefronts. More than half the CUs busy: as two K groups of four
+  // 64 x 64 wavefronts (2048^3: 14.5 us against 16.2; 11008 x 256 x 4096: 21.3 against 23.2); fewer: as 64 x 32
+  // wavefronts (1024^3: 8.4 against 9.1), where the K split or the 64 x 128 tile usually takes over anyway.
+  const long small = tiles(128, 128);
+  if (small <= 256) return small > 128 ? onebit::kTile128x128k2 : onebit::kTile128x128w8;
   return onebit::kTile128x128s;
 }
 
@@ -141,7 +145,8 @@ GemmPlan plan_gemm(int m, int n, int k) {
   const int forced_splits = g_split_k.load();
   const int tile = pick_tile(m, n);
   auto small_tile = [](int t) {
-    return t == onebit::kTile128x128s || t == onebit::kTile128x128w8 || t == onebit::kTile64x128;
+    return t == onebit::kTile128x128s || t == onebit::kTile128x128w8 || t == onebit::kTile64x128 ||
+           t == onebit::kTile128x128k2;
   };
   if (!small_tile(tile) || forced_splits >= 1) {
     int splits = forced_splits >= 1 ? forced_splits : 1;
@@ -156,7 +161,7 @@ GemmPlan plan_gemm(int m, int n, int k) {
     const int t = candidates[c];
     if (c == 1 && t == candidates[0]) break;
     const bool low = t == onebit::kTile64x128;
-    const double chunk_us = low ? 0.95 : 1.4;
+    const double chunk_us = low ? 0.95 : t == onebit::kTile128x128k2 ? 1.25 : 1.4;
     const double tiles = (double)((m + (low ? 63 : 127)) / (low ? 64 : 128)) * ((n + 127) / 128);
     for (int s : {1, 2, 3, 4, 6, 8, 12, 16}) {
       if (s > chunks) break;
@@ -356,9 +361,9 @@ int onebit_sparse_linear_prepared(const void* prepared, const void* x, const voi
   }
   switch (plan.rows_or_tile) {
     case onebit::kTile256x128w: case onebit::kTile128x128s: case onebit::kTile512x128w8: case onebit::kTile256x128w8:
-    case onebit::kTile128x128w8: case onebit::kTile64x128: break;
+    case onebit::kTile128x128w8: case onebit::kTile64x128: case onebit::kTile128x128k2: break;
     default:
-      return fail(ONEBIT_ERR_ARGUMENT, "tile configuration %d has no token-major variant (4, 6, 9, 10, 11, 12 have)",
+      return fail(ONEBIT_ERR_ARGUMENT, "tile configuration %d has no token-major variant (4, 6, 9, 10, 11, 12, 13 have)",
                   plan.rows_or_tile);
   }
   onebit::GemmArgs args{};

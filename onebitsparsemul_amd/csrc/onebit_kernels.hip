@@ -184,12 +184,14 @@ __device__ __forceinline__ int chunk_swizzle(int row) {
   return (BN >= 128) ? ((row & 3) << 2) : (((row >> 1) & 1) << 2);
 }
 
-template <int WM, int WN, int FM, int FN>
+// KG = 2: two groups of WM x WN wavefronts cover the same tile; group g multiplies K step g of every 64-row stage,
+// and the two partial tiles are added through LDS at the end (twice the wavefronts per SIMD for the same tile).
+template <int WM, int WN, int FM, int FN, int KG = 1>
 struct TileShape {
   static constexpr int BM = WM * FM * 32;
   static constexpr int BN = WN * FN * 32;
   static constexpr int CH = BN / 8;                       // 16-byte chunks per LDS row
-  static constexpr int NW = WM * WN;                      // wavefronts per workgroup
+  static constexpr int NW = WM * WN * KG;                 // wavefronts per workgroup
   static constexpr int NL = kStageK * CH / (64 * NW);     // chunk copies per thread per stage
   static constexpr int STAGE_BYTES = kStageK * BN * 2;
   static constexpr int LDS_B_BYTES = kStages * STAGE_BYTES;
@@ -198,6 +200,7 @@ struct TileShape {
   static_assert(NW == 4 || NW == 8, "four or eight wavefronts per workgroup");
   static_assert(kStageK * CH % (64 * NW) == 0, "the stage must divide into whole wavefront copies");
   static_assert(NL >= 1, "tile too narrow for the copy pattern");
+  static_assert(KG == 1 || (KG == 2 && WM * FM <= 4), "the second group's partial tile must fit the stage ring");
 };
 
 // XCD-aware tile order. Workgroup b runs on XCD b % 8, so XCD x is given a contiguous range of a tile list
@@ -414,16 +417,19 @@ __device__ __attribute__((aligned(16))) uint32_t g_zero16[4] = {0, 0, 0, 0};
 
 // TOKENS (with DMA only): the linear-layer form. p.b is x (p.n tokens x p.k, token-major), p.d is y (p.n tokens x
 // p.m), the epilogue is y = acc + bias; a tile column is a token.
-template <int WM, int WN, int FM, int FN, bool DMA, bool TOKENS = false>
-__global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmArgs p) {
+template <int WM, int WN, int FM, int FN, bool DMA, bool TOKENS = false, int KG = 1>
+__global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmArgs p) {
   static_assert(DMA || !TOKENS, "the token-major form uses the asynchronous copies");
-  using TS = TileShape<WM, WN, FM, FN>;
+  static_assert(DMA || KG == 1, "the two-group form uses the asynchronous copies");
+  using TS = TileShape<WM, WN, FM, FN, KG>;
   constexpr int BM = TS::BM, BN = TS::BN, CH = TS::CH, NL = TS::NL, NW = TS::NW;
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in a scalar register
-  const int wm = wave / WN, wn = wave % WN;
+  const int kg = KG == 2 ? wave / (WM * WN) : 0;   // K group of this wavefront
+  const int wave_in_group = KG == 2 ? wave % (WM * WN) : wave;
+  const int wm = wave_in_group / WN, wn = wave_in_group % WN;
   int tile_m, tile_n;
   tile_of_block<(NW == 8 ? 8 : 16)>(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
   const int row0 = tile_m * BM + wm * FM * 32;  // first row of this wavefront
@@ -481,6 +487,7 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
   const int chunk_begin = blockIdx.y * p.chunks_per_split;  // the launcher makes every split non-empty
   const int chunk_end = chunk_begin + p.chunks_per_split < chunks ? chunk_begin + p.chunks_per_split : chunks;
   char* const d_out = reinterpret_cast<char*>(p.d) + (size_t)blockIdx.y * p.m * p.n * (p.d_f16 ? 2 : 4);
+  const int row_limit = kg == 0 ? p.m : 0;  // the second K group hands its sums to the first and stores nothing
 
   if constexpr (DMA) {
     // ---- asynchronous copy pattern for B: NL 16-byte copies per thread per stage ----
@@ -571,75 +578,149 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm) a_frag_lds[fm] = a_lds + (wm * FM + fm) * kBlockBytes;
 
-    // Software pipeline. One K step (32 wide) is one scheduling region in which the SMFMACs of the step run
-    // while the B fragments and the expanded A of the next step are fetched. The workgroup barrier sits in the
-    // middle of each stage s: it publishes stage s+1 (read right after it) and frees the ring slot of stage s
-    // (all of its reads were issued in the first half), into which stage s+4 is then copied.
-    // Request order: A(0) B(0) B(1) B(2) B(3) | chunk c: mid s0: A(c+1) B(4c+4)  mid s1: B(4c+5)
-    //                                                     mid s2: B(4c+6)        mid s3: B(4c+7)
-    issue_a();
+    if constexpr (KG == 1) {
+      // Software pipeline. One K step (32 wide) is one scheduling region in which the SMFMACs of the step run
+      // while the B fragments and the expanded A of the next step are fetched. The workgroup barrier sits in the
+      // middle of each stage s: it publishes stage s+1 (read right after it) and frees the ring slot of stage s
+      // (all of its reads were issued in the first half), into which stage s+4 is then copied.
+      // Request order: A(0) B(0) B(1) B(2) B(3) | chunk c: mid s0: A(c+1) B(4c+4)  mid s1: B(4c+5)
+      //                                                     mid s2: B(4c+6)        mid s3: B(4c+7)
+      issue_a();
 #pragma unroll
-    for (int s = 0; s < kStages; ++s) issue_b(s);
+      for (int s = 0; s < kStages; ++s) issue_b(s);
 
-    AChunk a_cur[FM];
-    half16_t bv0[FN], bv1[FN];
-    half8_t av0[FM], av1[FM];
-    wait_vmcnt<3 * NL>();  // A(0) and B(0) have landed
-    __builtin_amdgcn_s_barrier();
+      AChunk a_cur[FM];
+      half16_t bv0[FN], bv1[FN];
+      half8_t av0[FM], av1[FM];
+      wait_vmcnt<3 * NL>();  // A(0) and B(0) have landed
+      __builtin_amdgcn_s_barrier();
 #pragma unroll
-    for (int fm = 0; fm < FM; ++fm) a_cur[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);
-    read_frags(0, 0, bv0);
-    expand_frags<0>(a_cur, one, av0);
+      for (int fm = 0; fm < FM; ++fm) a_cur[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);
+      read_frags(0, 0, bv0);
+      expand_frags<0>(a_cur, one, av0);
 
 #define ONEBIT_STAGE(S, WAITCNT, ISSUE_A)                                                                        \
-    {                                                                                                            \
-      read_frags((S), 1, bv1);                                                                                   \
-      expand_frags<2 * (S) + 1>(a_cur, one, av1);                                                                \
-      mfma_frags<2 * (S)>(a_cur, av0, bv0, acc);                                                                 \
-      interleave_region<FM, FN>();                                                                               \
-      __builtin_amdgcn_sched_barrier(0); /* keep the step's work inside its region */                           \
-      wait_vmcnt_lgkm0<(ONEBIT_EXP_WAIT_MODE == 1 ? 63 : ONEBIT_EXP_WAIT_MODE == 2 ? 0 : (WAITCNT))>(); /* copies of stage S+1 landed; this wavefront's reads of stage S returned */ \
-      if (!ONEBIT_EXP_NO_BARRIER) __builtin_amdgcn_s_barrier();                                                  \
-      if (ISSUE_A) issue_a();                                                                                    \
-      issue_b(S);                                                                                                \
-      read_frags(((S) + 1) % kStages, 0, bv0);                                                                   \
-    }
-
-    for (int kc = chunk_begin; kc < chunk_end; ++kc) {
-      // mid stage 0: waits for B(4c+1); newer requests: B(4c+2), B(4c+3)
-      ONEBIT_STAGE(0, 2 * NL, true)
-      expand_frags<2>(a_cur, one, av0);
-      mfma_frags<1>(a_cur, av1, bv1, acc);
-      interleave_region<FM, FN>();
-      __builtin_amdgcn_sched_barrier(0);
-      // mid stage 1: waits for B(4c+2); newer: B(4c+3), A(c+1), B(4c+4)
-      ONEBIT_STAGE(1, 2 * NL + NA, false)
-      expand_frags<4>(a_cur, one, av0);
-      mfma_frags<3>(a_cur, av1, bv1, acc);
-      interleave_region<FM, FN>();
-      __builtin_amdgcn_sched_barrier(0);
-      // mid stage 2: waits for B(4c+3); newer: A(c+1), B(4c+4), B(4c+5)
-      ONEBIT_STAGE(2, 2 * NL + NA, false)
-      expand_frags<6>(a_cur, one, av0);
-      mfma_frags<5>(a_cur, av1, bv1, acc);
-      interleave_region<FM, FN>();
-      __builtin_amdgcn_sched_barrier(0);
-      // mid stage 3: waits for B(4c+4), which is newer than A(c+1): the next chunk of A is readable after it
-      ONEBIT_STAGE(3, 2 * NL, false)
-      {
-        AChunk a_next[FM];
-#pragma unroll
-        for (int fm = 0; fm < FM; ++fm) a_next[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);
-        expand_frags<0>(a_next, one, av0);
-        mfma_frags<7>(a_cur, av1, bv1, acc);
-#pragma unroll
-        for (int fm = 0; fm < FM; ++fm) a_cur[fm] = a_next[fm];
+      {                                                                                                            \
+        read_frags((S), 1, bv1);                                                                                   \
+        expand_frags<2 * (S) + 1>(a_cur, one, av1);                                                                \
+        mfma_frags<2 * (S)>(a_cur, av0, bv0, acc);                                                                 \
+        interleave_region<FM, FN>();                                                                               \
+        __builtin_amdgcn_sched_barrier(0); /* keep the step's work inside its region */                           \
+        wait_vmcnt_lgkm0<(ONEBIT_EXP_WAIT_MODE == 1 ? 63 : ONEBIT_EXP_WAIT_MODE == 2 ? 0 : (WAITCNT))>(); /* copies of stage S+1 landed; this wavefront's reads of stage S returned */ \
+        if (!ONEBIT_EXP_NO_BARRIER) __builtin_amdgcn_s_barrier();                                                  \
+        if (ISSUE_A) issue_a();                                                                                    \
+        issue_b(S);                                                                                                \
+        read_frags(((S) + 1) % kStages, 0, bv0);                                                                   \
       }
-      interleave_region<FM, FN>();
-      __builtin_amdgcn_sched_barrier(0);
-    }
+
+      for (int kc = chunk_begin; kc < chunk_end; ++kc) {
+        // mid stage 0: waits for B(4c+1); newer requests: B(4c+2), B(4c+3)
+        ONEBIT_STAGE(0, 2 * NL, true)
+        expand_frags<2>(a_cur, one, av0);
+        mfma_frags<1>(a_cur, av1, bv1, acc);
+        interleave_region<FM, FN>();
+        __builtin_amdgcn_sched_barrier(0);
+        // mid stage 1: waits for B(4c+2); newer: B(4c+3), A(c+1), B(4c+4)
+        ONEBIT_STAGE(1, 2 * NL + NA, false)
+        expand_frags<4>(a_cur, one, av0);
+        mfma_frags<3>(a_cur, av1, bv1, acc);
+        interleave_region<FM, FN>();
+        __builtin_amdgcn_sched_barrier(0);
+        // mid stage 2: waits for B(4c+3); newer: A(c+1), B(4c+4), B(4c+5)
+        ONEBIT_STAGE(2, 2 * NL + NA, false)
+        expand_frags<6>(a_cur, one, av0);
+        mfma_frags<5>(a_cur, av1, bv1, acc);
+        interleave_region<FM, FN>();
+        __builtin_amdgcn_sched_barrier(0);
+        // mid stage 3: waits for B(4c+4), which is newer than A(c+1): the next chunk of A is readable after it
+        ONEBIT_STAGE(3, 2 * NL, false)
+        {
+          AChunk a_next[FM];
+#pragma unroll
+          for (int fm = 0; fm < FM; ++fm) a_next[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);
+          expand_frags<0>(a_next, one, av0);
+          mfma_frags<7>(a_cur, av1, bv1, acc);
+#pragma unroll
+          for (int fm = 0; fm < FM; ++fm) a_cur[fm] = a_next[fm];
+        }
+        interleave_region<FM, FN>();
+        __builtin_amdgcn_sched_barrier(0);
+      }
 #undef ONEBIT_STAGE
-    wait_vmcnt<0>();  // drain the copies issued past the end before the LDS is released
+      wait_vmcnt<0>();  // drain the copies issued past the end before the LDS is released
+    } else {
+      // Two K groups: this wavefront multiplies K step KGV of every stage. One barrier per stage: before it the
+      // wavefront waits for its fragments of stage S (read during stage S - 1) and for the copies of stage S + 1; after
+      // it the ring slot of stage S is free for stage S + 4 and stage S + 1 is readable. The fragments and the
+      // expanded signs of the next stage are fetched while the SMFMACs of this one run. Same request order and
+      // wait counts as the one-group pipeline.
+      auto run = [&](auto group_tag) __attribute__((always_inline)) {
+        constexpr int KGV = decltype(group_tag)::value;
+        issue_a();
+#pragma unroll
+        for (int s = 0; s < kStages; ++s) issue_b(s);
+        AChunk a_cur[FM];
+        half16_t bv_even[FN], bv_odd[FN];
+        half8_t av_even[FM], av_odd[FM];
+        wait_vmcnt<3 * NL>();  // A(0) and B(0) have landed
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm) a_cur[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);
+        read_frags(0, KGV, bv_even);
+        expand_frags<KGV>(a_cur, one, av_even);
+#define ONEBIT_GROUP_STAGE(S, WAITCNT, ISSUE_A, BV, AV, BV_NEXT, AV_NEXT)                                         \
+        {                                                                                                        \
+          wait_vmcnt_lgkm0<(WAITCNT)>();                                                                         \
+          __builtin_amdgcn_s_barrier();                                                                          \
+          if (ISSUE_A) issue_a();                                                                                \
+          issue_b(S);                                                                                            \
+          read_frags(((S) + 1) % kStages, KGV, BV_NEXT);                                                         \
+          if constexpr ((S) < kStages - 1) {                                                                     \
+            expand_frags<2 * ((S) + 1) + KGV>(a_cur, one, AV_NEXT);                                              \
+            mfma_frags<2 * (S) + KGV>(a_cur, AV, BV, acc);                                                       \
+          } else {                                                                                               \
+            AChunk a_next[FM];                                                                                   \
+            _Pragma("unroll") for (int fm = 0; fm < FM; ++fm) a_next[fm] = load_a_chunk_lds(a_frag_lds[fm], lane); \
+            expand_frags<KGV>(a_next, one, AV_NEXT);                                                             \
+            mfma_frags<2 * (S) + KGV>(a_cur, AV, BV, acc);                                                       \
+            _Pragma("unroll") for (int fm = 0; fm < FM; ++fm) a_cur[fm] = a_next[fm];                            \
+          }                                                                                                      \
+          __builtin_amdgcn_sched_barrier(0);                                                                     \
+        }
+        for (int kc = chunk_begin; kc < chunk_end; ++kc) {
+          ONEBIT_GROUP_STAGE(0, 2 * NL, true, bv_even, av_even, bv_odd, av_odd)
+          ONEBIT_GROUP_STAGE(1, 2 * NL + NA, false, bv_odd, av_odd, bv_even, av_even)
+          ONEBIT_GROUP_STAGE(2, 2 * NL + NA, false, bv_even, av_even, bv_odd, av_odd)
+          ONEBIT_GROUP_STAGE(3, 2 * NL, false, bv_odd, av_odd, bv_even, av_even)
+        }
+#undef ONEBIT_GROUP_STAGE
+        wait_vmcnt<0>();  // drain the copies issued past the end before the LDS is released
+      };
+      if (kg == 0) run(std::integral_constant<int, 0>{});
+      else run(std::integral_constant<int, 1>{});
+      // the second group's partial tile goes to the first through the stage ring, lane for lane
+      smfmac_drain();
+      __syncthreads();
+      float* const handover = reinterpret_cast<float*>(smem) + (size_t)wave_in_group * (FM * FN * 16 * 64) + lane;
+      if (kg == 1) {
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+          for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) handover[((fm * FN + fn) * 16 + v) * 64] = acc[fm][fn][v];
+      }
+      __syncthreads();
+      if (kg == 0) {
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+          for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[fm][fn][v] += handover[((fm * FN + fn) * 16 + v) * 64];
+      }
+      __syncthreads();  // the epilogue's scratch overlaps the handover area
+    }
   } else {
     // ---- generic path: any N, any K % 32 == 0, any alignment. One stage at a time, element copies. ----
     for (int kc = chunk_begin; kc < chunk_end; ++kc) {
@@ -723,7 +804,7 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
             const float4 lo = *reinterpret_cast<const float4*>(scratch + t * 128 + (((2 * j) ^ token_swizzle(t)) << 4));
             const float4 hi = *reinterpret_cast<const float4*>(scratch + t * 128 + (((2 * j + 1) ^ token_swizzle(t)) << 4));
             const float x[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-            if (token < p.n && row < p.m) {
+            if (token < p.n && row < row_limit) {
               float bias8[8];
               bias_vector(row, bias8, std::integral_constant<int, 8>{});
               half8_t out;
@@ -739,7 +820,7 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
             const int t = piece / 8, j = piece % 8;
             const int token = col0 + t, row = row_base + 4 * j;
             const float4 v4 = *reinterpret_cast<const float4*>(scratch + t * 128 + ((j ^ token_swizzle(t)) << 4));
-            if (token < p.n && row < p.m) {
+            if (token < p.n && row < row_limit) {
               float bias4[4];
               bias_vector(row, bias4, std::integral_constant<int, 4>{});
               *reinterpret_cast<float4*>(reinterpret_cast<float*>(d_out) + (size_t)token * p.m + row) =
@@ -759,7 +840,7 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int row = row0 + fm * 32 + 8 * (v / 4) + 4 * gb + (v % 4);
-          if (token < p.n && row < p.m) {
+          if (token < p.n && row < row_limit) {
             const float x = acc[fm][fn][v] + bias_of(row);
             const size_t o = (size_t)token * p.m + row;
             if (p.d_f16) reinterpret_cast<_Float16*>(d_out)[o] = (_Float16)x;
@@ -797,7 +878,7 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
             const float4 lo = *reinterpret_cast<const float4*>(scratch + r * WCOLS + c8);
             const float4 hi = *reinterpret_cast<const float4*>(scratch + r * WCOLS + c8 + 4);
             float x[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-            if (row < p.m && col < p.n && !(ONEBIT_EXP_NO_STORE && x[0] != 12345.f)) {
+            if (row < row_limit && col < p.n && !(ONEBIT_EXP_NO_STORE && x[0] != 12345.f)) {
               const size_t o = (size_t)row * p.n + col;
 #pragma unroll
               for (int j = 0; j < 8; ++j) x[j] = p.alpha * x[j];
@@ -829,7 +910,7 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
             const int row = row_base + r, col = col0 + c4;
             const float4 a4 = *reinterpret_cast<const float4*>(scratch + r * WCOLS + c4);
             float x[4] = {a4.x, a4.y, a4.z, a4.w};
-            if (row < p.m && col < p.n && !(ONEBIT_EXP_NO_STORE && x[0] != 12345.f)) {
+            if (row < row_limit && col < p.n && !(ONEBIT_EXP_NO_STORE && x[0] != 12345.f)) {
               const size_t o = (size_t)row * p.n + col;
 #pragma unroll
               for (int j = 0; j < 4; ++j) x[j] = p.alpha * x[j];
@@ -864,7 +945,7 @@ __global__ __launch_bounds__(64 * WM * WN, (FM * FN <= 8 ? 2 : 1)) void gemm_ker
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int row = row0 + fm * 32 + 8 * (v / 4) + row_lane + (v % 4);
-        if (row < p.m && col < p.n && !(ONEBIT_EXP_NO_STORE && acc[fm][fn][v] != 12345.f)) {
+        if (row < row_limit && col < p.n && !(ONEBIT_EXP_NO_STORE && acc[fm][fn][v] != 12345.f)) {
           const size_t o = (size_t)row * p.n + col;
           float x = p.alpha * acc[fm][fn][v];
           if (p.beta != 0.f) {
@@ -1367,13 +1448,13 @@ hipError_t launch_pack(const void* w, void* a, void* e, int m, int k, int prune,
   return hipGetLastError();
 }
 
-template <int WM, int WN, int FM, int FN, bool DMA, bool TOKENS = false>
+template <int WM, int WN, int FM, int FN, bool DMA, bool TOKENS = false, int KG = 1>
 static hipError_t launch_gemm_cfg(GemmArgs args, hipStream_t stream) {
-  using TS = TileShape<WM, WN, FM, FN>;
+  using TS = TileShape<WM, WN, FM, FN, KG>;
   args.tiles_m = (args.m + TS::BM - 1) / TS::BM;
   args.tiles_n = (args.n + TS::BN - 1) / TS::BN;
   const int lds = DMA ? TS::LDS_BYTES : TS::STAGE_BYTES;
-  auto kern = gemm_kernel<WM, WN, FM, FN, DMA, TOKENS>;
+  auto kern = gemm_kernel<WM, WN, FM, FN, DMA, TOKENS, KG>;
   // the dynamic-LDS limit is a per-device attribute of the kernel; threads that race here set the same value
   static std::atomic<bool> attr_done[64] = {};
   int device = 0;
@@ -1409,6 +1490,7 @@ static hipError_t launch_gemm_pass(GemmArgs args, int tile_config, hipStream_t s
     case kTile256x128w8: return launch_gemm_cfg<4, 2, 2, 2, true>(args, stream);
     case kTile128x128w8: return launch_gemm_cfg<2, 4, 2, 1, true>(args, stream);
     case kTile64x128: return launch_gemm_cfg<2, 2, 1, 2, true>(args, stream);
+    case kTile128x128k2: return launch_gemm_cfg<2, 2, 2, 2, true, false, 2>(args, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -1432,6 +1514,7 @@ hipError_t launch_gemm_tokens(GemmArgs args, int tile_config, hipStream_t stream
       case kTile256x128w8: return launch_gemm_cfg<4, 2, 2, 2, true, true>(a, stream);
       case kTile128x128w8: return launch_gemm_cfg<2, 4, 2, 1, true, true>(a, stream);
       case kTile64x128: return launch_gemm_cfg<2, 2, 1, 2, true, true>(a, stream);
+      case kTile128x128k2: return launch_gemm_cfg<2, 2, 2, 2, true, true, 2>(a, stream);
       default: return hipErrorInvalidValue;  // the tiles the automatic choice uses
     }
   };

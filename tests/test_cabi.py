@@ -132,7 +132,7 @@ def test_launch_plan_of_the_benchmark_shapes(_default_hooks):
     # the prefill shape has one 256 x 128 tile per CU: its eight-wavefront form (code 10)
     assert plan(4096, 2048, 4096) == dict(kernel="gemm_kernel", tile=10, splits=1, pad_b=False)
     # small squares: 128 x 128 / 64 x 128 tiles, no K split
-    assert plan(2048, 2048, 2048) == dict(kernel="gemm_kernel", tile=11, splits=1, pad_b=False)
+    assert plan(2048, 2048, 2048) == dict(kernel="gemm_kernel", tile=13, splits=1, pad_b=False)   # two K groups
     assert plan(512, 512, 512) == dict(kernel="gemm_kernel", tile=12, splits=1, pad_b=False)
     # decode shapes: the split-K kernel, row group by M
     for n in (1, 4, 16):
