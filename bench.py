@@ -129,6 +129,31 @@ def run_decode_rotating(m, k, n, launches=2000, copies=None):
                 frac_of_hbm_peak=nbytes / t_rot / 1e9 / HBM_PEAK_GBS)
 
 
+def run_layer_form(m, k, tokens, launches=1000):
+    """The linear layer's call y = x W^T + bias (x and y token-major) three ways, each inside a HIP graph: the
+    token-major kernel form, the plain kernel on operands that are already transposed (no bias), and the plain kernel
+    with the two transposes and the bias pass around it. The weight is the same every launch (cache-resident)."""
+    import torch
+    from onebitsparsemul_amd import _native, synthetic
+    a, meta = synthetic.make_weight(m, k, seed=5, device="cuda")
+    prep = _native.prepare(a, meta, m, k)
+    x = synthetic.make_b(tokens, k, seed=6, kind="normal", device="cuda")
+    bias = synthetic.make_b(1, m, seed=7, kind="normal", device="cuda").reshape(m)
+    b = x.T.contiguous()
+    d = torch.empty((m, tokens), dtype=torch.float16, device="cuda")
+    y = torch.empty((tokens, m), dtype=torch.float16, device="cuda")
+
+    def around(i):
+        _native.matmul_prepared(prep, x.T.contiguous(), d, m, tokens, k)
+        return d.T.contiguous() + bias
+
+    t_form = time_graph(lambda i: _native.linear_prepared(prep, x, y, m, k, bias=bias), launches)
+    t_plain = time_graph(lambda i: _native.matmul_prepared(prep, b, d, m, tokens, k), launches)
+    t_around = time_graph(around, max(50, launches // 4))
+    return dict(shape=f"{m}x{k}, {tokens} tokens", us_token_major_form=t_form * 1e6,
+                us_plain_kernel_pretransposed=t_plain * 1e6, us_plain_kernel_with_transposes_and_bias=t_around * 1e6)
+
+
 def cpu_baseline(w, operands, budget_s=12.0):
     """oracle (kind 'port'): decompress + dense fp32 torch.matmul on the host cores, on a row slab sized for
     about budget_s seconds; rate in the metric's unit (dense-equivalent TFLOP/s)."""
@@ -228,6 +253,8 @@ def main():
         line["decode_n16"] = run_decode_rotating(11008, 4096, 16)
         # the same kernel family where the weight is large enough for bandwidth, not latency, to set the time
         line["decode_n16_large"] = run_decode_rotating(28672, 8192, 16, launches=500)
+        # the linear layer's token-major form of the same kernels (decode and prefill sized)
+        line["layer_form"] = [run_layer_form(11008, 4096, 16), run_layer_form(4096, 4096, 2048, launches=200)]
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w, operands)
     print(json.dumps(line))
