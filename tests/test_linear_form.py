@@ -147,3 +147,31 @@ def test_layer_forward_with_bias(lead, x_dtype):
     store[1:] = x.reshape(-1).cuda().half()
     got2 = layer(store[1:].view(*lead, in_f))
     assert torch.equal(got2.cpu().float().reshape(-1, out_f), want)
+
+
+def test_linear_form_at_8192_identity_and_linearity():
+    """full size: x = I returns the transposed decompressed weight exactly; linearity on integer tokens, exact"""
+    m = k = tokens = 8192
+    a, meta = synthetic.make_weight(m, k, seed=0x0B5A0200)
+    dense = torch.from_numpy(oracle.decompress_operands(a.numpy(), meta.numpy(), m, k))
+    prep = _native.prepare(a.cuda(), meta.cuda(), m, k)
+    eye = torch.eye(k, dtype=torch.float16, device="cuda")
+    y = torch.empty((tokens, m), dtype=torch.float16, device="cuda")
+    _native.linear_prepared(prep, eye, y, m, k)
+    torch.cuda.synchronize()
+    del eye
+    assert torch.equal(y.to(torch.int8), dense.cuda().T)
+    x1 = synthetic.make_b(tokens, k, seed=1, kind="int", device="cuda")
+    x2 = synthetic.make_b(tokens, k, seed=2, kind="int", device="cuda")
+    outs = []
+    for x in (x1, x2, x1 + x2):
+        o = torch.empty((tokens, m), dtype=torch.float32, device="cuda")
+        _native.linear_prepared(prep, x, o, m, k)
+        outs.append(o)
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0] + outs[1], outs[2])
+    # and equal to the plain form on the transposed operand
+    d = torch.empty((m, tokens), dtype=torch.float32, device="cuda")
+    _native.matmul_prepared(prep, x1.T.contiguous(), d, m, tokens, k)
+    torch.cuda.synchronize()
+    assert torch.equal(d.T, outs[0])
