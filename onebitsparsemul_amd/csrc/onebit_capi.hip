@@ -128,51 +128,92 @@ int pick_tile(int m, int n) {
   return onebit::kTile128x128s;
 }
 
-// Tile and number of K splits of the main kernel. Few tiles and a long K leave most compute units idle and make
-// the time the length of one workgroup's K loop; a smaller tile (64 x 128) or a split of K fills the GPU, the split
-// at the price of a second launch and of writing and re-reading fp32 partial sums. In that regime (fewer than 256
-// tiles of 256 x 128) the choice comes from a cost model fitted to measurements on MI355X, in microseconds: one
-// workgroup's K loop takes 1.4 per 256-wide chunk with the 128 x 128 tile and 0.95 with the 64 x 128 tile, times
-// the rounds of one workgroup per CU; a split adds 5 for the second launch and the partial sums move at about 3 TB/s.
+// Tile and number of K splits of the main kernel. With at least 256 tiles of 512 x 128 the rules of pick_tile apply
+// (large tiles, no split). Below that, the time is rounds of resident workgroups times one workgroup's K loop, and the
+// choice among the tiles, and among splits of K that fill idle compute units at the price of a second launch and of
+// writing and re-reading fp32 partial sums, comes from a cost model fitted to measurements on MI355X (microseconds):
+//   K loop of one workgroup per 256-wide chunk with every slot of the GPU taken: 512 x 128: 3.8, 256 x 128 on eight
+//   wavefronts: 2.3, on four (two workgroups per CU): 3.9, 128 x 128 on four (two per CU): 2.4, as two K groups:
+//   1.2, as 64 x 32 wavefronts: 1.5, 64 x 128: 1.0;
+//   a round that fills only a fraction f of the slots is shorter: with one workgroup per CU 0.85 of a full round
+//   below f = 0.9; with two per CU 0.6 up to f = 0.5 (every workgroup has its CU to itself) and a full round above
+//   (some CUs hold two again); the two-K-group tile pays 1.5 per round for handing over the second group's sums;
+//   4 for launch, prologue and epilogue; a split adds 5 and moves (S + 1) partial results at about 4 TB/s.
+// Examples the model was checked against (measured, us): 4096 x 3072 x 4096: 512 x 128 57.0, 256 x 128 68.3;
+// 4096 x 1536 x 4096: 256 x 128 35.0, 128 x 128 38.9; 4096 x 384 x 11008: 64 x 128 40.2, 256 x 128 with four splits
+// 32.5; 11008 x 768 x 4096: 512 x 128 51.2, 256 x 128 65.5; 4096 x 128 x 4096: 64 x 128 with four splits 13.9,
+// unsplit 17.3.
 struct GemmPlan {
   int tile;
   int splits;
 };
 
+struct TileCost {
+  int tile, bm, bn;
+  int slots;        // workgroups resident on the GPU at once
+  double chunk_us;  // K loop of one workgroup per 256-wide chunk with every slot taken
+  double round_us;  // per round on top of the K loop
+  bool may_split;
+};
+const TileCost kTileCosts[] = {
+    {onebit::kTile512x128w8, 512, 128, 256, 3.8, 0.0, false}, {onebit::kTile256x128w8, 256, 128, 256, 2.3, 0.0, true},
+    {onebit::kTile256x128w, 256, 128, 512, 3.9, 0.0, false},  {onebit::kTile128x128s, 128, 128, 512, 2.4, 0.0, false},
+    {onebit::kTile128x128k2, 128, 128, 256, 1.2, 1.5, true}, {onebit::kTile128x128w8, 128, 128, 256, 1.5, 0.0, true},
+    {onebit::kTile64x128, 64, 128, 256, 1.0, 0.0, true},
+};
+
+double model_us(const TileCost& t, int m, int n, int chunks, int s) {
+  const long tiles = (long)((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn) * s;
+  const int per_split = (chunks + s - 1) / s;
+  const long full_rounds = tiles / t.slots;
+  const double f = (double)(tiles % t.slots) / t.slots;
+  double rounds = (double)full_rounds;
+  if (f > 0.0) rounds += t.slots == 256 ? (f > 0.9 ? 1.0 : 0.85) : (f <= 0.5 ? 0.6 : 1.0);
+  double us = 4.0 + (t.chunk_us * per_split + t.round_us) * rounds;
+  if (s > 1) us += 5.0 + (s + 1) * 4.0 * m * n / 4.0e6;
+  return us;
+}
+
 GemmPlan plan_gemm(int m, int n, int k) {
   const int chunks = (k + onebit::kChunkK - 1) / onebit::kChunkK;
   const int forced_tile = g_tile_config.load();
   const int forced_splits = g_split_k.load();
-  const int tile = pick_tile(m, n);
-  auto small_tile = [](int t) {
-    return t == onebit::kTile128x128s || t == onebit::kTile128x128w8 || t == onebit::kTile64x128 ||
-           t == onebit::kTile128x128k2;
-  };
-  if (!small_tile(tile) || forced_splits >= 1) {
+  const bool many_tiles = (long)((m + 511) / 512) * ((n + 127) / 128) >= 256;
+  if (many_tiles || forced_tile >= 0) {
+    // the rules of pick_tile (or the forced tile); a forced tile of the table may still be split by the model
+    const int tile = pick_tile(m, n);
     int splits = forced_splits >= 1 ? forced_splits : 1;
+    if (forced_splits < 1 && !many_tiles)
+      for (const TileCost& t : kTileCosts)
+        if (t.tile == tile && t.may_split) {
+          double best_us = 1e30;
+          for (int s : {1, 2, 3, 4, 6, 8, 12, 16}) {
+            if (s > chunks) break;
+            const double us = model_us(t, m, n, chunks, s);
+            if (us < best_us) best_us = us, splits = s;
+          }
+        }
     if (splits > chunks) splits = chunks;
     return GemmPlan{tile, splits};
   }
-  const double result_bytes = 4.0 * m * n;
-  GemmPlan best{tile, 1};
+  const int fixed_splits = forced_splits >= 1 ? (forced_splits > chunks ? chunks : forced_splits) : 0;
+  GemmPlan best{onebit::kTile128x128s, fixed_splits ? fixed_splits : 1};
   double best_us = 1e30;
-  const int candidates[2] = {tile, forced_tile >= 0 ? tile : (int)onebit::kTile64x128};
-  for (int c = 0; c < 2; ++c) {
-    const int t = candidates[c];
-    if (c == 1 && t == candidates[0]) break;
-    const bool low = t == onebit::kTile64x128;
-    const double chunk_us = low ? 0.95 : t == onebit::kTile128x128k2 ? 1.25 : 1.4;
-    const double tiles = (double)((m + (low ? 63 : 127)) / (low ? 64 : 128)) * ((n + 127) / 128);
+  auto consider = [&](const TileCost& t, int s) {
+    const double us = model_us(t, m, n, chunks, s);
+    if (us < best_us) {
+      best_us = us;
+      best = GemmPlan{t.tile, s};
+    }
+  };
+  for (const TileCost& t : kTileCosts) {
+    if (fixed_splits) {
+      consider(t, fixed_splits);
+      continue;
+    }
     for (int s : {1, 2, 3, 4, 6, 8, 12, 16}) {
-      if (s > chunks) break;
-      const int per_split = (chunks + s - 1) / s;
-      const double rounds = (double)(long)((tiles * s + 255) / 256);
-      double us = chunk_us * per_split * rounds;
-      if (s > 1) us += 5.0 + (s + 1) * result_bytes / 3.0e6;
-      if (us < best_us) {
-        best_us = us;
-        best = GemmPlan{t, s};
-      }
+      if (s > chunks || (s > 1 && !t.may_split)) break;
+      consider(t, s);
     }
   }
   return best;

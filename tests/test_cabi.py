@@ -146,6 +146,11 @@ def test_launch_plan_of_the_benchmark_shapes(_default_hooks):
     assert plan(28672, 64, 8192) == dict(kernel="skinny_kernel", rows=64)
     assert plan(65536, 64, 8192)["kernel"] == "gemm_kernel"      # from about 48k rows on the main kernel is faster
     assert plan(4096, 65, 4096)["kernel"] == "gemm_kernel"
+    # fewer than 256 tiles of 512 x 128: tile and split from the cost model
+    assert plan(4096, 3072, 4096) == dict(kernel="gemm_kernel", tile=9, splits=1, pad_b=False)    # 192 large tiles
+    assert plan(4096, 1536, 4096) == dict(kernel="gemm_kernel", tile=10, splits=1, pad_b=False)   # 192 of 256 x 128
+    assert plan(11008, 768, 4096)["tile"] == 9 and plan(28672, 192, 8192)["tile"] == 10
+    assert plan(4096, 384, 11008) == dict(kernel="gemm_kernel", tile=13, splits=2, pad_b=False)   # 96 tiles, 43 chunks
     # few tiles over a long K: split over workgroups; many tiles: never
     few = plan(4096, 128, 4096)
     assert few["kernel"] == "gemm_kernel" and few["splits"] > 1
