@@ -134,11 +134,11 @@ int pick_tile(int m, int n) {
 // writing and re-reading fp32 partial sums, comes from a cost model fitted to measurements on MI355X (microseconds):
 //   K loop of one workgroup per 256-wide chunk with every slot of the GPU taken: 512 x 128: 3.8, 256 x 128 on eight
 //   wavefronts: 2.3, on four (two workgroups per CU): 3.9, 128 x 128 on four (two per CU): 2.4, as two K groups:
-//   1.2, as 64 x 32 wavefronts: 1.5, 64 x 128: 1.0;
+//   1.2, as 64 x 32 wavefronts: 1.5, 64 x 128: 1.0, as two K groups: 0.88;
 //   a round that fills only a fraction f of the slots is shorter: with one workgroup per CU 0.85 of a full round
 //   below f = 0.9; with two per CU 0.6 up to f = 0.5 (every workgroup has its CU to itself) and a full round above
-//   (some CUs hold two again); the two-K-group tile pays 1.5 per round for handing over the second group's sums;
-//   4 for launch, prologue and epilogue; a split adds 5 and moves (S + 1) partial results at about 4 TB/s.
+//   (some CUs hold two again); the two-K-group tiles pay 1.5 and 1.0 per round for handing over the second group's sums;
+//   4 for launch, prologue and epilogue; a split adds 5 and moves (S + 1) partial results at about 5 TB/s.
 // Examples the model was checked against (measured, us): 4096 x 3072 x 4096: 512 x 128 57.0, 256 x 128 68.3;
 // 4096 x 1536 x 4096: 256 x 128 35.0, 128 x 128 38.9; 4096 x 384 x 11008: 64 x 128 40.2, 256 x 128 with four splits
 // 32.5; 11008 x 768 x 4096: 512 x 128 51.2, 256 x 128 65.5; 4096 x 128 x 4096: 64 x 128 with four splits 13.9,
@@ -159,7 +159,7 @@ const TileCost kTileCosts[] = {
     {onebit::kTile512x128w8, 512, 128, 256, 3.8, 0.0, false}, {onebit::kTile256x128w8, 256, 128, 256, 2.3, 0.0, true},
     {onebit::kTile256x128w, 256, 128, 512, 3.9, 0.0, false},  {onebit::kTile128x128s, 128, 128, 512, 2.4, 0.0, false},
     {onebit::kTile128x128k2, 128, 128, 256, 1.2, 1.5, true}, {onebit::kTile128x128w8, 128, 128, 256, 1.5, 0.0, true},
-    {onebit::kTile64x128, 64, 128, 256, 1.0, 0.0, true},
+    {onebit::kTile64x128, 64, 128, 256, 1.0, 0.0, true},      {onebit::kTile64x128k2, 64, 128, 256, 0.88, 1.0, true},
 };
 
 double model_us(const TileCost& t, int m, int n, int chunks, int s) {
@@ -170,7 +170,7 @@ double model_us(const TileCost& t, int m, int n, int chunks, int s) {
   double rounds = (double)full_rounds;
   if (f > 0.0) rounds += t.slots == 256 ? (f > 0.9 ? 1.0 : 0.85) : (f <= 0.5 ? 0.6 : 1.0);
   double us = 4.0 + (t.chunk_us * per_split + t.round_us) * rounds;
-  if (s > 1) us += 5.0 + (s + 1) * 4.0 * m * n / 4.0e6;
+  if (s > 1) us += 5.0 + (s + 1) * 4.0 * m * n / 5.0e6;
   return us;
 }
 
@@ -402,9 +402,9 @@ int onebit_sparse_linear_prepared(const void* prepared, const void* x, const voi
   }
   switch (plan.rows_or_tile) {
     case onebit::kTile256x128w: case onebit::kTile128x128s: case onebit::kTile512x128w8: case onebit::kTile256x128w8:
-    case onebit::kTile128x128w8: case onebit::kTile64x128: case onebit::kTile128x128k2: break;
+    case onebit::kTile128x128w8: case onebit::kTile64x128: case onebit::kTile128x128k2: case onebit::kTile64x128k2: break;
     default:
-      return fail(ONEBIT_ERR_ARGUMENT, "tile configuration %d has no token-major variant (4, 6, 9, 10, 11, 12, 13 have)",
+      return fail(ONEBIT_ERR_ARGUMENT, "tile configuration %d has no token-major variant (4, 6, 9 ... 14 have)",
                   plan.rows_or_tile);
   }
   onebit::GemmArgs args{};

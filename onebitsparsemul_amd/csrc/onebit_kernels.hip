@@ -1491,6 +1491,7 @@ static hipError_t launch_gemm_pass(GemmArgs args, int tile_config, hipStream_t s
     case kTile128x128w8: return launch_gemm_cfg<2, 4, 2, 1, true>(args, stream);
     case kTile64x128: return launch_gemm_cfg<2, 2, 1, 2, true>(args, stream);
     case kTile128x128k2: return launch_gemm_cfg<2, 2, 2, 2, true, false, 2>(args, stream);
+    case kTile64x128k2: return launch_gemm_cfg<2, 2, 1, 2, true, false, 2>(args, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -1515,6 +1516,7 @@ hipError_t launch_gemm_tokens(GemmArgs args, int tile_config, hipStream_t stream
       case kTile128x128w8: return launch_gemm_cfg<2, 4, 2, 1, true, true>(a, stream);
       case kTile64x128: return launch_gemm_cfg<2, 2, 1, 2, true, true>(a, stream);
       case kTile128x128k2: return launch_gemm_cfg<2, 2, 2, 2, true, true, 2>(a, stream);
+      case kTile64x128k2: return launch_gemm_cfg<2, 2, 1, 2, true, true, 2>(a, stream);
       default: return hipErrorInvalidValue;  // the tiles the automatic choice uses
     }
   };

@@ -48,13 +48,13 @@ struct SkinnyArgs {
   int bias_f16;
 };
 
-enum TileConfig { kTile512x128 = 0, kTile256x128 = 1, kTile128x128 = 2, kTile256x256 = 3, kTile256x128w = 4, kTile512x128t = 5, kTile128x128s = 6, kTile256x64 = 7, kTile256x256w8 = 8, kTile512x128w8 = 9, kTile256x128w8 = 10, kTile128x128w8 = 11, kTile64x128 = 12, kTile128x128k2 = 13, kTileAuto = -1 };
+enum TileConfig { kTile512x128 = 0, kTile256x128 = 1, kTile128x128 = 2, kTile256x256 = 3, kTile256x128w = 4, kTile512x128t = 5, kTile128x128s = 6, kTile256x64 = 7, kTile256x256w8 = 8, kTile512x128w8 = 9, kTile256x128w8 = 10, kTile128x128w8 = 11, kTile64x128 = 12, kTile128x128k2 = 13, kTile64x128k2 = 14, kTileAuto = -1 };
 
 hipError_t launch_prepare(const void* a, const void* e, void* prep, int m, int k, int layout, hipStream_t stream);
 hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream);
 // The linear layer's form of the main kernel: b is x (n tokens x k, token-major, 16-byte aligned), d is y (n tokens x
 // m), y = x W^T + bias; c, alpha, beta and the padded copy of B are not used, splits / chunks_per_split / split_ws as in
-// launch_gemm. Tiles 4, 6, 9, 10, 11, 12, 13.
+// launch_gemm. Tiles 4, 6, 9, 10, 11, 12, 13, 14.
 hipError_t launch_gemm_tokens(GemmArgs args, int tile_config, hipStream_t stream);
 // dense fp16 (m x k) -> one-bit values `a` and metadata `e`; prune != 0 applies the 2:4 magnitude mask first
 hipError_t launch_pack(const void* w, void* a, void* e, int m, int k, int prune, int layout, hipStream_t stream);

@@ -151,6 +151,7 @@ def test_launch_plan_of_the_benchmark_shapes(_default_hooks):
     assert plan(4096, 1536, 4096) == dict(kernel="gemm_kernel", tile=10, splits=1, pad_b=False)   # 192 of 256 x 128
     assert plan(11008, 768, 4096)["tile"] == 9 and plan(28672, 192, 8192)["tile"] == 10
     assert plan(4096, 384, 11008) == dict(kernel="gemm_kernel", tile=13, splits=2, pad_b=False)   # 96 tiles, 43 chunks
+    assert plan(4096, 512, 4096) == dict(kernel="gemm_kernel", tile=14, splits=1, pad_b=False)    # 64 x 128, two K groups
     # few tiles over a long K: split over workgroups; many tiles: never
     few = plan(4096, 128, 4096)
     assert few["kernel"] == "gemm_kernel" and few["splits"] > 1
