@@ -105,8 +105,31 @@ def _require_cuda(*tensors):
     return dev
 
 
+class _on_device:
+    """Make `dev` the current device for the duration of a library call; free when it already is (the usual case:
+    entering torch.cuda.device() costs more than the call it guards)."""
+
+    def __init__(self, dev):
+        self._guard = None if dev.index == torch.cuda.current_device() else torch.cuda.device(dev)
+
+    def __enter__(self):
+        if self._guard is not None:
+            self._guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self._guard is not None:
+            self._guard.__exit__(*exc)
+        return False
+
+
 def prepared_bytes(m, k):
     return lib().onebit_sparse_prepared_bytes(m, k)
+
+
+def _prepared_bytes_fast(m, k):
+    """onebit_sparse_prepared_bytes without the library call (hot path of the per-call checks): one 1536-byte
+    block per 32 rows and 256 columns."""
+    return ((m + 31) // 32) * ((k + 255) // 256) * 1536
 
 
 def prepare(a, meta, m, k, layout=META_REFERENCE):
@@ -115,7 +138,7 @@ def prepare(a, meta, m, k, layout=META_REFERENCE):
     if a.numel() * a.element_size() != m * k // 16 or meta.numel() * meta.element_size() != m * k // 8:
         raise ValueError("operand sizes do not match m, k")
     out = torch.empty(prepared_bytes(m, k), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _check(lib().onebit_sparse_prepare(a.data_ptr(), meta.data_ptr(), m, k, layout, out.data_ptr(), _stream(a)))
     return out
 
@@ -126,9 +149,9 @@ def matmul_prepared(prepared, b, d, m, n, k, c=None, alpha=1.0, beta=0.0):
         raise ValueError("B must be float16 of shape (k, n)")
     if tuple(d.shape) != (m, n) or (c is not None and tuple(c.shape) != (m, n)):
         raise ValueError("C / D must have shape (m, n)")
-    if prepared.numel() != prepared_bytes(m, k):
+    if prepared.numel() != _prepared_bytes_fast(m, k):
         raise ValueError("prepared operand does not match m, k")
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _check(lib().onebit_sparse_matmul_prepared(
             prepared.data_ptr(), b.data_ptr(), c.data_ptr() if c is not None else None, d.data_ptr(), m, n, k,
             alpha, beta, _dtype_code(c) if c is not None else F32, _dtype_code(d), _stream(b)))
@@ -143,9 +166,9 @@ def linear_prepared(prepared, x, y, m, k, bias=None):
         raise ValueError("x must be float16 of shape (tokens, k)")
     if tuple(y.shape) != (tokens, m) or (bias is not None and tuple(bias.shape) != (m,)):
         raise ValueError("y must have shape (tokens, m) and bias (m,)")
-    if prepared.numel() != prepared_bytes(m, k):
+    if prepared.numel() != _prepared_bytes_fast(m, k):
         raise ValueError("prepared operand does not match m, k")
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _check(lib().onebit_sparse_linear_prepared(
             prepared.data_ptr(), x.data_ptr(), bias.data_ptr() if bias is not None else None, y.data_ptr(), tokens, m, k,
             _dtype_code(bias) if bias is not None else F16, _dtype_code(y), _stream(x)))
@@ -156,7 +179,7 @@ def matmul_ex(a, b, meta, d, m, n, k, c=None, alpha=1.0, beta=0.0, layout=META_R
     dev = _require_cuda(a, b, meta, d, c)
     if b.dtype != torch.float16 or tuple(b.shape) != (k, n):
         raise ValueError("B must be float16 of shape (k, n)")
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _check(lib().onebit_sparse_matmul_ex(
             a.data_ptr(), b.data_ptr(), c.data_ptr() if c is not None else None, d.data_ptr(), meta.data_ptr(), m, n,
             k, alpha, beta, _dtype_code(c) if c is not None else F32, _dtype_code(d), layout, _stream(b)))
@@ -166,7 +189,7 @@ def matmul_ex(a, b, meta, d, m, n, k, c=None, alpha=1.0, beta=0.0, layout=META_R
 def matmul_legacy(a, b, c, d, meta, m, n, k):
     """The 8-argument entry point: fp32 C/D, alpha = 1, beta = 0, default stream."""
     dev = _require_cuda(a, b, c, d, meta)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         lib().onebit_sparse_matmul(a.data_ptr(), b.data_ptr(), c.data_ptr(), d.data_ptr(), meta.data_ptr(), m, n, k)
     return d
 
@@ -208,7 +231,7 @@ def pack_weight(weight, prune=True, layout=META_REFERENCE):
     m, k = weight.shape
     a = torch.empty((k // 2, m // 8), dtype=torch.uint8, device=dev)
     meta = torch.empty((m, k // 16), dtype=torch.int16, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _check(lib().onebit_sparse_pack(weight.data_ptr(), m, k, 1 if prune else 0, a.data_ptr(), meta.data_ptr(), layout,
                                         _stream(weight)))
     return a, meta

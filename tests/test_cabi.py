@@ -184,3 +184,8 @@ def test_describe_launch_validates():
     out = (ctypes.c_int * 4)()
     assert lib.onebit_sparse_describe_launch(60, 8, 32, 1, out) == 1
     assert lib.onebit_sparse_describe_launch(64, 8, 32, 1, None) == 1
+
+
+def test_python_side_size_formula_matches_the_library():
+    for m, k in ((64, 32), (64, 256), (96, 288), (4096, 11008), (28672, 8192)):
+        assert _native._prepared_bytes_fast(m, k) == _native.prepared_bytes(m, k)
