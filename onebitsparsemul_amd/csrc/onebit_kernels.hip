@@ -1090,6 +1090,14 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
     if (TOKENS) {
       // offsets at or past n * k * 2 (tokens >= n) fall outside the descriptor and read as zero; K positions at or
       // past k are sent there too (the launcher checks that 64 * k * 2 stays well below 2^32)
+      if (k_base + IMG_ROWS <= k_rows) {
+        // the image's whole K range exists (wave-uniform test): lane offsets that do not change from image to image
+        // plus a scalar offset; the range check looks at the lane offset alone, which is what sends tokens >= n to zero
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          v[i] = buffer_load16(b_buffer, token_load_base + i * token_load_step, (uint32_t)k_base * 2u);
+        return;
+      }
       const bool inside = k_base + 8 * piece_lane < k_rows;
       const uint32_t first = token_load_base + (uint32_t)k_base * 2u;
 #pragma unroll
