@@ -102,36 +102,10 @@ int check_dtype(int c_dtype, int d_dtype) {
   return ONEBIT_OK;
 }
 
-int pick_tile(int m, int n) {
-  const int forced = g_tile_config.load();
-  if (forced >= 0) return forced;
-  // Largest tile that still gives every CU its share of workgroups (measured on MI355X at the sustained clock):
-  // 512 x 128 with eight wavefronts (one workgroup per CU) from 256 tiles on - 8192^3: 2.2 PF, 4096^3: 2.03 PF
-  // against 1.91 PF for 256 x 128 - unless its last round of 256 would be mostly empty (11008 x 2048 x 4096: 352
-  // tiles, 117 us against 102 us for 256 x 128); 256 x 128 with four wavefronts from 256 tiles on (8192 x 1024 x
-  // 8192: 76 us against 83 us for 128 x 128); 128 x 128 (64 x 64 per wavefront, two workgroups per CU) below that.
-  auto tiles = [&](int bm, int bn) { return (long)((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
-  const long big = tiles(512, 128);
-  // its rounds of 256 workgroups at least 77 % full (5120^3, 78 %: 140 us against 151; 6144^3, 75 %: 255 against 234)
-  if (big >= 256 && big * 100 >= ((big + 255) / 256) * 256 * 77) return onebit::kTile512x128w8;
-  // With at most one workgroup per CU the eight-wavefront forms of the small tiles run two wavefronts per SIMD
-  // instead of one: 256 x 128 (4096 x 2048 x 4096: 42.4 us against 46.3), 128 x 128 (2048^3: 14.9 against 15.6,
-  // 1024^3: 8.4 against 9.2, 512^3: 5.9 against 6.6).
-  const long mid = tiles(256, 128);
-  if (mid >= 512) return onebit::kTile256x128w;
-  if (mid >= 256) return onebit::kTile256x128w8;
-  // at most one 128 x 128 workgroup per CU: eight wavefronts. More than half the CUs busy: as two K groups of four
-  // 64 x 64 wavefronts (2048^3: 14.5 us against 16.2; 11008 x 256 x 4096: 21.3 against 23.2); fewer: as 64 x 32
-  // wavefronts (1024^3: 8.4 against 9.1), where the K split or the 64 x 128 tile usually takes over anyway.
-  const long small = tiles(128, 128);
-  if (small <= 256) return small > 128 ? onebit::kTile128x128k2 : onebit::kTile128x128w8;
-  return onebit::kTile128x128s;
-}
-
-// Tile and number of K splits of the main kernel. With at least 256 tiles of 512 x 128 the rules of pick_tile apply
-// (large tiles, no split). Below that, the time is rounds of resident workgroups times one workgroup's K loop, and the
-// choice among the tiles, and among splits of K that fill idle compute units at the price of a second launch and of
-// writing and re-reading fp32 partial sums, comes from a cost model fitted to measurements on MI355X (microseconds):
+// Tile and number of K splits of the main kernel. The time is rounds of resident workgroups times one workgroup's K
+// loop; the choice among the tiles, and among splits of K that fill idle compute units at the price of a second launch
+// and of writing and re-reading fp32 partial sums, comes from a cost model fitted to measurements on MI355X
+// (microseconds):
 //   K loop of one workgroup per 256-wide chunk with every slot of the GPU taken: 512 x 128: 3.8, 256 x 128 on eight
 //   wavefronts: 2.3, on four (two workgroups per CU): 3.9, 128 x 128 on four (two per CU): 2.4, as two K groups:
 //   1.2, as 64 x 32 wavefronts: 1.5, 64 x 128: 1.0, as two K groups: 0.88;
@@ -178,14 +152,12 @@ GemmPlan plan_gemm(int m, int n, int k) {
   const int chunks = (k + onebit::kChunkK - 1) / onebit::kChunkK;
   const int forced_tile = g_tile_config.load();
   const int forced_splits = g_split_k.load();
-  const bool many_tiles = (long)((m + 511) / 512) * ((n + 127) / 128) >= 256;
-  if (many_tiles || forced_tile >= 0) {
-    // the rules of pick_tile (or the forced tile); a forced tile of the table may still be split by the model
-    const int tile = pick_tile(m, n);
+  if (forced_tile >= 0) {
+    // a forced tile of the table may still be split by the model
     int splits = forced_splits >= 1 ? forced_splits : 1;
-    if (forced_splits < 1 && !many_tiles)
+    if (forced_splits < 1)
       for (const TileCost& t : kTileCosts)
-        if (t.tile == tile && t.may_split) {
+        if (t.tile == forced_tile && t.may_split) {
           double best_us = 1e30;
           for (int s : {1, 2, 3, 4, 6, 8, 12, 16}) {
             if (s > chunks) break;
@@ -194,7 +166,7 @@ GemmPlan plan_gemm(int m, int n, int k) {
           }
         }
     if (splits > chunks) splits = chunks;
-    return GemmPlan{tile, splits};
+    return GemmPlan{forced_tile, splits};
   }
   const int fixed_splits = forced_splits >= 1 ? (forced_splits > chunks ? chunks : forced_splits) : 0;
   GemmPlan best{onebit::kTile128x128s, fixed_splits ? fixed_splits : 1};
