@@ -487,7 +487,11 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
   const int chunk_begin = blockIdx.y * p.chunks_per_split;  // the launcher makes every split non-empty
   const int chunk_end = chunk_begin + p.chunks_per_split < chunks ? chunk_begin + p.chunks_per_split : chunks;
   char* const d_out = reinterpret_cast<char*>(p.d) + (size_t)blockIdx.y * p.m * p.n * (p.d_f16 ? 2 : 4);
-  const int row_limit = kg == 0 ? p.m : 0;  // the second K group hands its sums to the first and stores nothing
+  // Two K groups: with an even number of row fragments each group finishes half of them (it hands the other half of
+  // its sums to the other group); otherwise the second group hands everything to the first and stores nothing.
+  constexpr bool kSplitEpilogue = KG == 2 && FM % 2 == 0;
+  const int row_limit = (kg == 0 || kSplitEpilogue) ? p.m : 0;
+  auto finishes = [&](int fm) __attribute__((always_inline)) { return !kSplitEpilogue || (fm >= FM / 2) == (kg == 1); };
 
   if constexpr (DMA) {
     // ---- asynchronous copy pattern for B: NL 16-byte copies per thread per stage ----
@@ -698,26 +702,54 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
       };
       if (kg == 0) run(std::integral_constant<int, 0>{});
       else run(std::integral_constant<int, 1>{});
-      // the second group's partial tile goes to the first through the stage ring, lane for lane
       smfmac_drain();
-      __syncthreads();
-      float* const handover = reinterpret_cast<float*>(smem) + (size_t)wave_in_group * (FM * FN * 16 * 64) + lane;
-      if (kg == 1) {
+      __syncthreads();  // the stage ring is free
+      if constexpr (kSplitEpilogue) {
+        // each group keeps half of the row fragments and passes its sums for the other half through the ring, lane for
+        // lane: group 0 finishes fragments [0, FM / 2), group 1 the rest
+        constexpr int HALF = FM / 2, PER_WAVE = HALF * FN * 16 * 64;
+        float* const given = reinterpret_cast<float*>(smem) + (size_t)wave * PER_WAVE + lane;
+        const float* const taken =
+            reinterpret_cast<const float*>(smem) + (size_t)(wave_in_group + (1 - kg) * WM * WN) * PER_WAVE + lane;
 #pragma unroll
-        for (int fm = 0; fm < FM; ++fm)
-#pragma unroll
-          for (int fn = 0; fn < FN; ++fn)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) handover[((fm * FN + fn) * 16 + v) * 64] = acc[fm][fn][v];
-      }
-      __syncthreads();
-      if (kg == 0) {
-#pragma unroll
-        for (int fm = 0; fm < FM; ++fm)
+        for (int fm = 0; fm < HALF; ++fm)
 #pragma unroll
           for (int fn = 0; fn < FN; ++fn)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[fm][fn][v] += handover[((fm * FN + fn) * 16 + v) * 64];
+            for (int v = 0; v < 16; ++v) {
+              if (kg == 0) given[((fm * FN + fn) * 16 + v) * 64] = acc[HALF + fm][fn][v];
+              else given[((fm * FN + fn) * 16 + v) * 64] = acc[fm][fn][v];
+            }
+        __syncthreads();
+#pragma unroll
+        for (int fm = 0; fm < HALF; ++fm)
+#pragma unroll
+          for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              if (kg == 0) acc[fm][fn][v] += taken[((fm * FN + fn) * 16 + v) * 64];
+              else acc[HALF + fm][fn][v] += taken[((fm * FN + fn) * 16 + v) * 64];
+            }
+      } else {
+        // the second group's partial tile goes to the first, lane for lane
+        float* const handover = reinterpret_cast<float*>(smem) + (size_t)wave_in_group * (FM * FN * 16 * 64) + lane;
+        if (kg == 1) {
+#pragma unroll
+          for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+            for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+              for (int v = 0; v < 16; ++v) handover[((fm * FN + fn) * 16 + v) * 64] = acc[fm][fn][v];
+        }
+        __syncthreads();
+        if (kg == 0) {
+#pragma unroll
+          for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+            for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+              for (int v = 0; v < 16; ++v) acc[fm][fn][v] += handover[((fm * FN + fn) * 16 + v) * 64];
+        }
       }
       __syncthreads();  // the epilogue's scratch overlaps the handover area
     }
@@ -788,6 +820,7 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
       char* scratch = smem + wave * (WCOLS * 128);
 #pragma unroll
       for (int fm = 0; fm < FM; ++fm) {
+        if (!finishes(fm)) continue;  // the other K group stores this fragment
 #pragma unroll
         for (int fn = 0; fn < FN; ++fn)
 #pragma unroll
@@ -833,7 +866,8 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
     }
     // y not 16-byte aligned: one element per accumulator register
 #pragma unroll
-    for (int fm = 0; fm < FM; ++fm)
+    for (int fm = 0; fm < FM; ++fm) {
+      if (!finishes(fm)) continue;  // the other K group stores this fragment
 #pragma unroll
       for (int fn = 0; fn < FN; ++fn) {
         const int token = col0 + fn * 32 + token_lane;
@@ -848,6 +882,7 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
           }
         }
       }
+    }
     return;
   }
   // ---- epilogue: D = alpha * acc + beta * C (csrc/kernel.h:27-31), fp16 (RNE) or fp32 output ----
@@ -862,6 +897,7 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
       const int col_lane = lane & 31, row_lane = 4 * (lane >> 5);
 #pragma unroll
       for (int fm = 0; fm < FM; ++fm) {
+        if (!finishes(fm)) continue;  // the other K group stores this fragment
 #pragma unroll
         for (int fn = 0; fn < FN; ++fn)
 #pragma unroll
@@ -939,6 +975,7 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
   const int row_lane = 4 * (lane >> 5);
 #pragma unroll
   for (int fm = 0; fm < FM; ++fm) {
+    if (!finishes(fm)) continue;  // the other K group stores this fragment
 #pragma unroll
     for (int fn = 0; fn < FN; ++fn) {
       const int col = col0 + fn * 32 + col_lane;
