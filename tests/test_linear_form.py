@@ -175,3 +175,33 @@ def test_linear_form_at_8192_identity_and_linearity():
     _native.matmul_prepared(prep, x1.T.contiguous(), d, m, tokens, k)
     torch.cuda.synchronize()
     assert torch.equal(d.T, outs[0])
+
+
+@pytest.mark.parametrize("tokens,m,k", [(16, 1024, 2048), (300, 512, 512), (128, 256, 8192)])
+def test_linear_form_in_a_hip_graph(tokens, m, k):
+    """the layer's call captured in a HIP graph (after one eager call on the capture stream, which sizes the K-split
+    buffer): every replay, with new activations written in between, equals the eager result; split-K kernel, main
+    kernel, and its K split over workgroups"""
+    a, meta = synthetic.make_weight(m, k, seed=m + tokens)
+    prep = _native.prepare(a.cuda(), meta.cuda(), m, k)
+    bias = synthetic.make_b(1, m, seed=3, kind="int").reshape(m).cuda()
+    x = torch.zeros((tokens, k), dtype=torch.float16, device="cuda")
+    y = torch.zeros((tokens, m), dtype=torch.float32, device="cuda")
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        _native.linear_prepared(prep, x, y, m, k, bias=bias)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            _native.linear_prepared(prep, x, y, m, k, bias=bias)
+    for replay in range(4):
+        values = synthetic.make_b(tokens, k, seed=100 + replay, kind="int").cuda()
+        x.copy_(values)
+        y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = torch.empty_like(y)
+        _native.linear_prepared(prep, values, eager, m, k, bias=bias)
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager) and bool(torch.isfinite(y).all())
