@@ -111,7 +111,7 @@ int check_dtype(int c_dtype, int d_dtype) {
 //   1.2, as 64 x 32 wavefronts: 1.5, 64 x 128: 1.0, as two K groups: 0.88;
 //   a round that fills only a fraction f of the slots is shorter: with one workgroup per CU 0.85 of a full round
 //   below f = 0.9; with two per CU 0.6 up to f = 0.5 (every workgroup has its CU to itself) and a full round above
-//   (some CUs hold two again); the two-K-group tiles pay 1.5 and 1.0 per round for handing over the second group's sums;
+//   (some CUs hold two again); the two-K-group tiles pay 1.5 and 1.0 per round for exchanging the groups' sums;
 //   4 for launch, prologue and epilogue; a split adds 5 and moves (S + 1) partial results at about 5 TB/s.
 // Examples the model was checked against (measured, us): 4096 x 3072 x 4096: 512 x 128 57.0, 256 x 128 68.3;
 // 4096 x 1536 x 4096: 256 x 128 35.0, 128 x 128 38.9; 4096 x 384 x 11008: 64 x 128 40.2, 256 x 128 with four splits
@@ -124,7 +124,7 @@ struct GemmPlan {
 
 struct TileCost {
   int tile, bm, bn;
-  int slots;        // workgroups resident on the GPU at once
+  int slots;        // workgroups resident on the GPU at once (256 CUs: the model is for MI355X, like the kernels)
   double chunk_us;  // K loop of one workgroup per 256-wide chunk with every slot taken
   double round_us;  // per round on top of the K loop
   bool may_split;
