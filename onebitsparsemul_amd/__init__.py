@@ -179,6 +179,8 @@ class BinaryLinear_2_4(nn.Module):
         if self._prepared is None or self._prepared.buffer.device != x.device:
             self._prepared = PreparedWeight(self.packed_binary_sparse.to(x.device), self.meta.to(x.device))
         lead = x.shape[:-1]
+        if x.numel() == 0:  # an empty batch: nothing to launch
+            return x.new_zeros(*lead, self.outfeatures)
         tokens = x.reshape(-1, self.infeatures).to(torch.float16).contiguous()
         bias = self.bias
         if bias is not None and (bias.dtype not in (torch.float16, torch.float32) or bias.device != x.device):

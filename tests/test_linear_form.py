@@ -205,3 +205,14 @@ def test_linear_form_in_a_hip_graph(tokens, m, k):
         _native.linear_prepared(prep, values, eager, m, k, bias=bias)
         torch.cuda.synchronize()
         assert torch.equal(y, eager) and bool(torch.isfinite(y).all())
+
+
+def test_layer_forward_of_an_empty_batch():
+    import onebitsparsemul_amd as ob
+    layer = ob.BinaryLinear_2_4(64, 128)
+    layer.pack(torch.randn(128, 64).half())
+    layer = layer.cuda()
+    out = layer(torch.empty((0, 64), dtype=torch.float16, device="cuda"))
+    assert tuple(out.shape) == (0, 128) and out.dtype == torch.float16
+    out = layer(torch.empty((2, 0, 64), dtype=torch.float16, device="cuda"))
+    assert tuple(out.shape) == (2, 0, 128)
