@@ -69,6 +69,11 @@ def time_graph(fn, launches, warmup=20):
     import torch
     side = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
+    # The operands of fn were produced, and blocks of the caching allocator freed, by work queued on the current
+    # stream: without this wait the warm-up launches below run concurrently with that work, read operands that are not
+    # written yet and write their output into memory that a still-pending kernel of the current stream may own
+    # (a freed temporary the allocator handed out again).
+    side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
         # warm up on the capture stream: the library keeps its K-split and padded-B buffers per stream and may only
         # allocate them outside a capture

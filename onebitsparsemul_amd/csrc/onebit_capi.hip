@@ -73,8 +73,18 @@ struct DeviceState {
 };
 DeviceState g_dev[kMaxDevices];
 
-int grow(void** ptr, size_t* have, size_t need) {
+// Grows a library-owned buffer. Growing frees the old memory after a device synchronization: a HIP graph captured
+// earlier on this stream still holds the old address and must be captured again after a larger call. Inside a stream
+// capture neither the synchronization nor the allocation is possible, so a call that would have to grow there is
+// refused instead of invalidating the capture.
+int grow(void** ptr, size_t* have, size_t need, hipStream_t stream) {
   if (need <= *have) return ONEBIT_OK;
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  ONEBIT_HIP(hipStreamIsCapturing(stream, &capture));
+  if (capture != hipStreamCaptureStatusNone)
+    return fail(ONEBIT_ERR_ARGUMENT,
+                "a library-owned buffer would have to grow to %zu bytes while the stream is being captured: run the "
+                "call once outside the capture first, or use the non-allocating entry point", need);
   if (*ptr) {
     // earlier work on any stream may still read the old buffer
     ONEBIT_HIP(hipDeviceSynchronize());
@@ -226,8 +236,15 @@ LaunchPlan choose_launch(int m, int n, int k, bool b_16_byte_aligned) {
   return plan;
 }
 
+// Workspace of one call that the caller cannot let allocate: `base` is this device's copy of the file-scope array
+// g_static_scratch (see onebit_sparse_matmul_prepared_static), `bytes` its size.
+struct FixedScratch {
+  unsigned char* base;
+  size_t bytes;
+};
+
 int matmul_prepared_impl(const void* prepared, const void* b, const void* c, void* d, int m, int n, int k, float alpha,
-                         float beta, int c_dtype, int d_dtype, hipStream_t stream) {
+                         float beta, int c_dtype, int d_dtype, hipStream_t stream, const FixedScratch* fixed = nullptr) {
   if (!prepared || !b || !d) return fail(ONEBIT_ERR_ARGUMENT, "null operand pointer");
   if (beta != 0.f && !c) return fail(ONEBIT_ERR_ARGUMENT, "c must not be null when beta != 0");
   const int kc_total = (k + onebit::kChunkK - 1) / onebit::kChunkK;
@@ -262,23 +279,41 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
   const int splits = plan.splits;
   const bool pad_b = plan.pad_b != 0;
   if (splits > 1 || pad_b) {
+    size_t split_bytes = 0, pad_bytes = 0;
+    if (splits > 1) {
+      const int cps = (kc_total + splits - 1) / splits;
+      args.chunks_per_split = cps;
+      args.splits = (kc_total + cps - 1) / cps;  // every split non-empty
+      split_bytes = (size_t)args.splits * m * n * sizeof(float);
+    }
+    if (pad_b) pad_bytes = (size_t)k * ((size_t)(n + 7) / 8 * 8) * sizeof(_Float16);
+    if (fixed) {
+      // partial sums first, the padded copy of B behind them on the next 256-byte boundary; both are written in
+      // full by this call's own kernels before they are read, so nothing has to start at zero
+      const size_t pad_at = (split_bytes + 255) & ~size_t(255);
+      if (pad_at + pad_bytes > fixed->bytes)
+        return fail(ONEBIT_ERR_ARGUMENT,
+                    "this shape needs %zu bytes of scratch (%d K splits of %d x %d fp32 partial sums, %zu bytes of "
+                    "padded B); the static workspace of the non-allocating entry point holds %zu",
+                    pad_at + pad_bytes, splits > 1 ? args.splits : 0, m, n, pad_bytes, fixed->bytes);
+      if (splits > 1) args.split_ws = reinterpret_cast<float*>(fixed->base);
+      if (pad_b) args.b_pad = reinterpret_cast<_Float16*>(fixed->base + pad_at);
+      ONEBIT_HIP(onebit::launch_gemm(args, tile, stream));
+      return ONEBIT_OK;
+    }
     int device = 0;
     ONEBIT_HIP(hipGetDevice(&device));
     if (device < 0 || device >= kMaxDevices) return fail(ONEBIT_ERR_ARGUMENT, "device ordinal %d not supported", device);
     DeviceState& st = g_dev[device];
     std::lock_guard<std::mutex> lock(st.mu);
     if (splits > 1) {
-      const int cps = (kc_total + splits - 1) / splits;
-      args.chunks_per_split = cps;
-      args.splits = (kc_total + cps - 1) / cps;  // every split non-empty
       Buffer& ws = st.split_ws[stream];
-      if (int rc = grow(&ws.ptr, &ws.bytes, (size_t)args.splits * m * n * sizeof(float)); rc != ONEBIT_OK) return rc;
+      if (int rc = grow(&ws.ptr, &ws.bytes, split_bytes, stream); rc != ONEBIT_OK) return rc;
       args.split_ws = static_cast<float*>(ws.ptr);
     }
     if (pad_b) {
       Buffer& pb = st.b_pad[stream];
-      const size_t ldb = (size_t)(n + 7) / 8 * 8;
-      if (int rc = grow(&pb.ptr, &pb.bytes, (size_t)k * ldb * sizeof(_Float16)); rc != ONEBIT_OK) return rc;
+      if (int rc = grow(&pb.ptr, &pb.bytes, pad_bytes, stream); rc != ONEBIT_OK) return rc;
       args.b_pad = static_cast<_Float16*>(pb.ptr);
     }
     ONEBIT_HIP(onebit::launch_gemm(args, tile, stream));
@@ -399,7 +434,7 @@ int onebit_sparse_linear_prepared(const void* prepared, const void* x, const voi
     args.chunks_per_split = cps;
     args.splits = (kc_total + cps - 1) / cps;  // every split non-empty
     Buffer& ws = st.split_ws[s];
-    if (int rc = grow(&ws.ptr, &ws.bytes, (size_t)args.splits * m * tokens * sizeof(float)); rc != ONEBIT_OK) return rc;
+    if (int rc = grow(&ws.ptr, &ws.bytes, (size_t)args.splits * m * tokens * sizeof(float), s); rc != ONEBIT_OK) return rc;
     args.split_ws = static_cast<float*>(ws.ptr);
     ONEBIT_HIP(onebit::launch_gemm_tokens(args, plan.rows_or_tile, s));
     return ONEBIT_OK;
@@ -435,6 +470,11 @@ int onebit_sparse_matmul_ex(const void* a, const void* b, const void* c, void* d
           break;
         }
       if (!prep) {
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        ONEBIT_HIP(hipStreamIsCapturing(s, &capture));
+        if (capture != hipStreamCaptureStatusNone)
+          return fail(ONEBIT_ERR_ARGUMENT, "a weight that is not in the cache yet cannot be added while the stream is "
+                                           "being captured: run the call once outside the capture first");
         if ((int)ds.weight_cache.size() >= cache_entries) {  // evict the least recently used entry
           size_t victim = 0;
           for (size_t i = 1; i < ds.weight_cache.size(); ++i)
@@ -466,7 +506,7 @@ int onebit_sparse_matmul_ex(const void* a, const void* b, const void* c, void* d
   {
     std::lock_guard<std::mutex> lock(ds.mu);
     Buffer& own = ds.prep[s];
-    if (int rc = grow(&own.ptr, &own.bytes, onebit::prepared_bytes(m, k))) return rc;
+    if (int rc = grow(&own.ptr, &own.bytes, onebit::prepared_bytes(m, k), s)) return rc;
     prep = own.ptr;
   }
   ONEBIT_HIP(onebit::launch_prepare(a, e, prep, m, k, meta_layout, s));
