@@ -76,6 +76,23 @@ int onebit_sparse_matmul_prepared(const void *prepared, const void *b, const voi
                                   float alpha, float beta, int c_dtype, int d_dtype, void *stream);
 
 /*
+ * The prepared product for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc. It has no counterpart in the reference. Same arguments, kernels and results
+ * as onebit_sparse_matmul_prepared; the only difference is where the two internal buffers live that some shapes need
+ * (fp32 partial sums when K is split over workgroups, a copy of B with padded rows when B's rows are not 16-byte
+ * aligned): in a fixed array of ONEBIT_STATIC_SCRATCH_BYTES bytes that is part of the library's device code, of
+ * which every GPU the library runs on holds one copy until the process ends. The call never calls hipMalloc, hipFree
+ * or any allocating routine. A shape whose buffers do not fit is refused with ONEBIT_ERR_ARGUMENT and a message
+ * that names the sizes (onebit_sparse_describe_launch tells which shapes need buffers: plan[2] > 1 or plan[3] = 1).
+ * The buffers are written in full by the call's own kernels before they are read, so the contents a previous call
+ * left behind do no harm; but every call on one GPU uses the same array, so two such calls that overlap in time on
+ * one GPU (different streams, or different threads) race. Calls on one stream are ordered and safe.
+ */
+#define ONEBIT_STATIC_SCRATCH_BYTES (64u << 20)
+int onebit_sparse_matmul_prepared_static(const void *prepared, const void *b, const void *c, void *d, int m, int n,
+                                         int k, float alpha, float beta, int c_dtype, int d_dtype, void *stream);
+
+/*
  * Linear-layer form of the prepared product, for the forward pass of BinaryLinear_2_4
  * (onebit_sparse_mul/__init__.py:116-128), whose activations are token-major:
  *     y[t][r] = sum over k of W[r][k] * x[t][k]  (+ bias[r] when bias is not NULL)

@@ -14,7 +14,7 @@ META_REFERENCE, META_CUTLASS, META_LOGICAL = 0, 1, 2
 
 EXPORTS = (
     "onebit_sparse_matmul", "onebit_sparse_matmul_ex", "onebit_sparse_prepared_bytes", "onebit_sparse_prepare",
-    "onebit_sparse_matmul_prepared", "onebit_sparse_linear_prepared", "onebit_sparse_pack", "onebit_sparse_last_error", "onebit_sparse_set_tile_config",
+    "onebit_sparse_matmul_prepared", "onebit_sparse_matmul_prepared_static", "onebit_sparse_linear_prepared", "onebit_sparse_pack", "onebit_sparse_last_error", "onebit_sparse_set_tile_config",
     "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_set_split_k", "onebit_sparse_set_pad_b", "onebit_sparse_describe_launch", "onebit_sparse_set_weight_cache", "onebit_sparse_clear_weight_cache",
     "onebit_sparse_measure_smfmac_rate", "onebit_sparse_device_info",
 )
@@ -39,6 +39,8 @@ def lib():
         L.onebit_sparse_prepare.argtypes = [vp, vp, i32, i32, i32, vp, vp]
         L.onebit_sparse_matmul_prepared.restype = i32
         L.onebit_sparse_matmul_prepared.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, i32, vp]
+        L.onebit_sparse_matmul_prepared_static.restype = i32
+        L.onebit_sparse_matmul_prepared_static.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, i32, vp]
         L.onebit_sparse_linear_prepared.restype = i32
         L.onebit_sparse_linear_prepared.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp]
         L.onebit_sparse_pack.restype = i32
@@ -143,7 +145,12 @@ def prepare(a, meta, m, k, layout=META_REFERENCE):
     return out
 
 
-def matmul_prepared(prepared, b, d, m, n, k, c=None, alpha=1.0, beta=0.0):
+STATIC_SCRATCH_BYTES = 64 << 20
+
+
+def matmul_prepared(prepared, b, d, m, n, k, c=None, alpha=1.0, beta=0.0, static_scratch=False):
+    """D = alpha * A * B + beta * C on the prepared weight. static_scratch=True takes the entry point that never
+    allocates device memory (its internal buffers live in a fixed array of STATIC_SCRATCH_BYTES)."""
     dev = _require_cuda(prepared, b, d, c)
     if b.dtype != torch.float16 or tuple(b.shape) != (k, n):
         raise ValueError("B must be float16 of shape (k, n)")
@@ -151,8 +158,9 @@ def matmul_prepared(prepared, b, d, m, n, k, c=None, alpha=1.0, beta=0.0):
         raise ValueError("C / D must have shape (m, n)")
     if prepared.numel() != _prepared_bytes_fast(m, k):
         raise ValueError("prepared operand does not match m, k")
+    entry = lib().onebit_sparse_matmul_prepared_static if static_scratch else lib().onebit_sparse_matmul_prepared
     with _on_device(dev):
-        _check(lib().onebit_sparse_matmul_prepared(
+        _check(entry(
             prepared.data_ptr(), b.data_ptr(), c.data_ptr() if c is not None else None, d.data_ptr(), m, n, k,
             alpha, beta, _dtype_code(c) if c is not None else F32, _dtype_code(d), _stream(b)))
     return d

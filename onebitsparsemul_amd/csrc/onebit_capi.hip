@@ -43,6 +43,13 @@ int fail(int code, const char* fmt, ...) {
 
 constexpr int kMaxDevices = 64;
 
+// Workspace of onebit_sparse_matmul_prepared_static: device memory that exists from the moment the code object is
+// loaded, so that entry point never allocates. Every GPU the library runs on holds its own copy at its own address
+// until the process ends. In host code the name is only a handle for hipGetSymbolAddress; kernels and copies use the
+// per-device address kept in DeviceState::static_scratch.
+constexpr size_t kStaticScratchBytes = ONEBIT_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
+
 // Library-owned device memory. Grow-only, one buffer per device and stream (calls on one stream are ordered, calls
 // on different streams must not share a buffer), freed at process exit by the runtime.
 struct Buffer {
@@ -70,6 +77,8 @@ struct DeviceState {
   };
   std::vector<CachedWeight> weight_cache;
   unsigned long use_counter = 0;
+  // this device's address of g_static_scratch (null until the first non-allocating call on the device)
+  unsigned char* static_scratch = nullptr;
 };
 DeviceState g_dev[kMaxDevices];
 
@@ -382,6 +391,31 @@ int onebit_sparse_matmul_prepared(const void* prepared, const void* b, const voi
   if (int rc = check_shape(m, n, k)) return rc;
   if (int rc = check_dtype(c_dtype, d_dtype)) return rc;
   return matmul_prepared_impl(prepared, b, c, d, m, n, k, alpha, beta, c_dtype, d_dtype, static_cast<hipStream_t>(stream));
+}
+
+int onebit_sparse_matmul_prepared_static(const void* prepared, const void* b, const void* c, void* d, int m, int n, int k,
+                                         float alpha, float beta, int c_dtype, int d_dtype, void* stream) {
+  g_last_error.clear();
+  if (int rc = check_shape(m, n, k)) return rc;
+  if (int rc = check_dtype(c_dtype, d_dtype)) return rc;
+  int device = 0;
+  ONEBIT_HIP(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) return fail(ONEBIT_ERR_ARGUMENT, "device ordinal %d not supported", device);
+  DeviceState& st = g_dev[device];
+  FixedScratch fixed{nullptr, kStaticScratchBytes};
+  {
+    std::lock_guard<std::mutex> lock(st.mu);
+    if (!st.static_scratch) {
+      // once per device, with that device current: the address of this device's copy of the array
+      void* address = nullptr;
+      ONEBIT_HIP(hipGetSymbolAddress(&address, HIP_SYMBOL(g_static_scratch)));
+      if (!address) return fail(ONEBIT_ERR_HIP, "hipGetSymbolAddress returned a null address for the static workspace");
+      st.static_scratch = static_cast<unsigned char*>(address);
+    }
+    fixed.base = st.static_scratch;
+  }
+  return matmul_prepared_impl(prepared, b, c, d, m, n, k, alpha, beta, c_dtype, d_dtype,
+                              static_cast<hipStream_t>(stream), &fixed);
 }
 
 int onebit_sparse_linear_prepared(const void* prepared, const void* x, const void* bias, void* y, int tokens, int m,
