@@ -302,6 +302,32 @@ def test_split_k_kernel_large_m_row_groups(m, k, n, rows):
     assert np.array_equal(y.cpu().numpy(), exact.T)
 
 
+@pytest.mark.parametrize("m,k,ns", [(8192, 28672, (40, 48, 64)), (4096, 16384, (16,)), (2048, 20480, (32,))])
+def test_split_k_kernel_long_k(m, k, ns):
+    """long K (64 to 112 chunks of 256) through the split-K kernel's 16-, 32- and 64-column images with 32- and
+    64-row workgroups, through the main kernel with its planned K split, and through the token-major form of both:
+    bit-exact against the oracle on integer operands"""
+    a, meta = synthetic.make_weight(m, k, seed=m + k)
+    dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
+    prep = _native.prepare(a.cuda(), meta.cuda(), m, k)
+    for n in ns:
+        bi = synthetic.make_b(k, n, seed=n, kind="int")
+        exact = oracle.blas_matmul(dense, bi.numpy(), dtype=np.float32)  # integers: exact in fp32 BLAS too
+        bd = bi.cuda()
+        xd = bd.T.contiguous()
+        for rows, skinny in ((32, True), (64, True), (-1, False)):
+            _native.set_skinny_rows(rows)
+            _native.set_skinny_enabled(skinny)
+            d = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+            _native.matmul_prepared(prep, bd, d, m, n, k)
+            y = torch.full((n, m), float("nan"), dtype=torch.float32, device="cuda")
+            _native.linear_prepared(prep, xd, y, m, k)
+            torch.cuda.synchronize()
+            assert np.array_equal(d.cpu().numpy(), exact), (n, rows, skinny)
+            assert np.array_equal(y.cpu().numpy(), exact.T), (n, rows, skinny, "token-major")
+    del dense
+
+
 def test_config3_split_k_is_deterministic_and_reusable():
     m, k, n = 4096, 11008, 16
     a, meta = synthetic.make_weight(m, k, seed=5)
