@@ -895,19 +895,41 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
       constexpr int WCOLS = FN * 32;                   // columns of the wavefront's tile
       float* scratch = reinterpret_cast<float*>(smem) + wave * (32 * WCOLS);
       const int col_lane = lane & 31, row_lane = 4 * (lane >> 5);
+      // The pieces of C that a lane will need for one 32-row block are requested together, before the block's sums
+      // travel through the scratch, so that one memory latency per block is paid instead of one per piece.
+      const bool use_c = p.beta != 0.f;
 #pragma unroll
       for (int fm = 0; fm < FM; ++fm) {
         if (!finishes(fm)) continue;  // the other K group stores this fragment
-#pragma unroll
-        for (int fn = 0; fn < FN; ++fn)
-#pragma unroll
-          for (int v = 0; v < 16; ++v)
-            scratch[(8 * (v / 4) + row_lane + (v % 4)) * WCOLS + fn * 32 + col_lane] = acc[fm][fn][v];
         const int row_base = row0 + fm * 32;
         if (p.d_f16) {
           constexpr int PER_ROW = WCOLS / 8;           // 16-byte pieces (8 halves) per row
+          constexpr int ITERS = 32 * PER_ROW / 64;
+          uint32_t c_raw[ITERS][8];                    // fp16 C: one 16-byte load per piece (words 0-3); fp32 C: two
 #pragma unroll
-          for (int it = 0; it < 32 * PER_ROW / 64; ++it) {
+          for (int it = 0; it < ITERS; ++it) {
+            const int piece = it * 64 + lane;
+            const int row = row_base + piece / PER_ROW, col = col0 + (piece % PER_ROW) * 8;
+            u32x4_t lo = u32x4_t{0, 0, 0, 0}, hi = u32x4_t{0, 0, 0, 0};
+            if (use_c && row < row_limit && col < p.n) {
+              const size_t o = (size_t)row * p.n + col;
+              if (p.c_f16) {
+                lo = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const _Float16*>(p.c) + o);
+              } else {
+                lo = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const float*>(p.c) + o);
+                hi = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const float*>(p.c) + o + 4);
+              }
+            }
+            c_raw[it][0] = lo.x; c_raw[it][1] = lo.y; c_raw[it][2] = lo.z; c_raw[it][3] = lo.w;
+            c_raw[it][4] = hi.x; c_raw[it][5] = hi.y; c_raw[it][6] = hi.z; c_raw[it][7] = hi.w;
+          }
+#pragma unroll
+          for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+              scratch[(8 * (v / 4) + row_lane + (v % 4)) * WCOLS + fn * 32 + col_lane] = acc[fm][fn][v];
+#pragma unroll
+          for (int it = 0; it < ITERS; ++it) {
             const int piece = it * 64 + lane;
             const int r = piece / PER_ROW, c8 = (piece % PER_ROW) * 8;
             const int row = row_base + r, col = col0 + c8;
@@ -918,17 +940,15 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
               const size_t o = (size_t)row * p.n + col;
 #pragma unroll
               for (int j = 0; j < 8; ++j) x[j] = p.alpha * x[j];
-              if (p.beta != 0.f) {
+              if (use_c) {
                 if (p.c_f16) {
-                  const half8_t cv = *reinterpret_cast<const half8_t*>(reinterpret_cast<const _Float16*>(p.c) + o);
+                  const half8_t cv =
+                      __builtin_bit_cast(half8_t, u32x4_t{c_raw[it][0], c_raw[it][1], c_raw[it][2], c_raw[it][3]});
 #pragma unroll
                   for (int j = 0; j < 8; ++j) x[j] = x[j] + p.beta * (float)cv[j];
                 } else {
-                  const float4 c0 = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.c) + o);
-                  const float4 c1 = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.c) + o + 4);
-                  const float cv[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
 #pragma unroll
-                  for (int j = 0; j < 8; ++j) x[j] = x[j] + p.beta * cv[j];
+                  for (int j = 0; j < 8; ++j) x[j] = x[j] + p.beta * __builtin_bit_cast(float, c_raw[it][j]);
                 }
               }
               half8_t out;
@@ -939,8 +959,31 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
           }
         } else {
           constexpr int PER_ROW = WCOLS / 4;           // 16-byte pieces (4 floats) per row
+          constexpr int ITERS = 32 * PER_ROW / 64;
+          uint32_t c_raw[ITERS][4];                    // fp32 C: one 16-byte load per piece; fp16 C: one 8-byte load
 #pragma unroll
-          for (int it = 0; it < 32 * PER_ROW / 64; ++it) {
+          for (int it = 0; it < ITERS; ++it) {
+            const int piece = it * 64 + lane;
+            const int row = row_base + piece / PER_ROW, col = col0 + (piece % PER_ROW) * 4;
+            u32x4_t lo = u32x4_t{0, 0, 0, 0};
+            if (use_c && row < row_limit && col < p.n) {
+              const size_t o = (size_t)row * p.n + col;
+              if (p.c_f16) {
+                const u32x2_t t = *reinterpret_cast<const u32x2_t*>(reinterpret_cast<const _Float16*>(p.c) + o);
+                lo.x = t.x; lo.y = t.y;
+              } else {
+                lo = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const float*>(p.c) + o);
+              }
+            }
+            c_raw[it][0] = lo.x; c_raw[it][1] = lo.y; c_raw[it][2] = lo.z; c_raw[it][3] = lo.w;
+          }
+#pragma unroll
+          for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+              scratch[(8 * (v / 4) + row_lane + (v % 4)) * WCOLS + fn * 32 + col_lane] = acc[fm][fn][v];
+#pragma unroll
+          for (int it = 0; it < ITERS; ++it) {
             const int piece = it * 64 + lane;
             const int r = piece / PER_ROW, c4 = (piece % PER_ROW) * 4;
             const int row = row_base + r, col = col0 + c4;
@@ -950,16 +993,14 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
               const size_t o = (size_t)row * p.n + col;
 #pragma unroll
               for (int j = 0; j < 4; ++j) x[j] = p.alpha * x[j];
-              if (p.beta != 0.f) {
+              if (use_c) {
                 if (p.c_f16) {
-                  const _Float16* cp = reinterpret_cast<const _Float16*>(p.c) + o;
+                  const half4_t cv = __builtin_bit_cast(half4_t, u32x2_t{c_raw[it][0], c_raw[it][1]});
 #pragma unroll
-                  for (int j = 0; j < 4; ++j) x[j] = x[j] + p.beta * (float)cp[j];
+                  for (int j = 0; j < 4; ++j) x[j] = x[j] + p.beta * (float)cv[j];
                 } else {
-                  const float4 c0 = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.c) + o);
-                  const float cv[4] = {c0.x, c0.y, c0.z, c0.w};
 #pragma unroll
-                  for (int j = 0; j < 4; ++j) x[j] = x[j] + p.beta * cv[j];
+                  for (int j = 0; j < 4; ++j) x[j] = x[j] + p.beta * __builtin_bit_cast(float, c_raw[it][j]);
                 }
               }
               *reinterpret_cast<float4*>(reinterpret_cast<float*>(d_out) + o) = float4{x[0], x[1], x[2], x[3]};
