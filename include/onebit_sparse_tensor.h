@@ -58,8 +58,10 @@ void onebit_sparse_matmul(void *a, void *b, void *c, void *d, void *e, int m, in
  * (csrc/kernel.h:27-31), fp16 or fp32 c and d, metadata layout, explicit stream (hipStream_t passed as
  * void*, NULL = default stream). Returns a status code and never exits.
  * The reordered copy of (a, e) is written on every call to a library-owned workspace kept per device and per
- * stream (grown with a device synchronization when a larger weight arrives): calls on different streams may
- * overlap; the prepared form below skips the reorder pass and allocates nothing.
+ * stream (grown with a device synchronization when a larger weight arrives; the old buffer is freed, so a HIP graph
+ * captured before a larger call on the same stream must be captured again, and a call that would have to grow a
+ * buffer while its stream is being captured is refused): calls on different streams may overlap; the prepared form
+ * below skips the reorder pass.
  */
 int onebit_sparse_matmul_ex(const void *a, const void *b, const void *c, void *d, const void *e, int m, int n, int k,
                             float alpha, float beta, int c_dtype, int d_dtype, int meta_layout, void *stream);
@@ -118,7 +120,7 @@ const char *onebit_sparse_last_error(void);
 /* Tuning / test hooks: force a tile configuration of the main kernel (-1 = automatic) and choose whether
  * shapes with n <= 32 (n <= 64 when m <= 40960) use the split-K kernel (1, default) or the main kernel (0).
  * Tile codes 0-14 are the TileConfig values of csrc/onebit_launch.h (the linear-layer form has 4, 6, 9-14).
- * Process-wide. */
+ * These five hooks act on the calling thread only: the calls that thread makes afterwards. */
 void onebit_sparse_set_tile_config(int tile_config);
 void onebit_sparse_set_skinny_enabled(int enabled);
 /* Weight rows one workgroup of the split-K kernel covers: 32, 64 or 128; <= 0 = automatic. */
@@ -145,8 +147,15 @@ void onebit_sparse_set_pad_b(int enabled);
 int onebit_sparse_set_weight_cache(int entries);
 int onebit_sparse_clear_weight_cache(void);
 
+/* Frees every library-owned buffer (the reordered operands of the one-call entry points, K-split partial sums and
+ * padded copies of B, kept per device and per stream and otherwise held until the process ends) after synchronizing
+ * the devices that hold any. The weight cache and the static workspace are not touched. Not inside a stream capture;
+ * HIP graphs captured earlier must not be replayed afterwards. No counterpart in the reference (its launcher allocates
+ * and frees a workspace on every call, csrc/kernel_lib.cu:73-76). */
+int onebit_sparse_release_buffers(void);
+
 /* Diagnostic, no counterpart in the reference, host-only (touches no GPU): what a prepared call of this shape would
- * launch under the current hooks. plan[0] = 1 for the split-K kernel (n <= 64), 0 for the main kernel; plan[1] =
+ * launch under the calling thread's hooks on a GPU with 256 compute units (calls plan for the device they run on). plan[0] = 1 for the split-K kernel (n <= 64), 0 for the main kernel; plan[1] =
  * weight rows per workgroup (split-K kernel) or the tile code (main kernel); plan[2] = K splits over workgroups
  * (main kernel, 1 = none); plan[3] = 1 if B is read through a padded copy. */
 int onebit_sparse_describe_launch(int m, int n, int k, int b_16_byte_aligned, int *plan);

@@ -135,12 +135,20 @@ class BinaryLinear_2_4(nn.Module):
     """1-bit 2:4 sparse linear layer: y = x @ W.T (+ bias when one has been assigned), W (outfeatures, infeatures)
     stored at 1.5 bits per weight. Reference: onebit_sparse_mul/__init__.py:101-145."""
 
-    def __init__(self, infeatures: int, outfeatures: int):
+    def __init__(self, infeatures: int, outfeatures: int, out_dtype=None):
+        """out_dtype: dtype of the kernel's result. None (default): float16 for float16 activations (the sums are
+        accumulated in fp32 and rounded once; a sum of infeatures/2 terms of +-x can exceed float16's range for large
+        activations) and float32 for every other activation dtype, so that the only precision loss is the cast of x
+        to float16. torch.float32 returns the reference layer's fp32 product for float16 activations as well
+        (onebit_sparse_mul/__init__.py:12-14: cuda_binary_mul returns an fp32 C)."""
         super().__init__()
         if infeatures % 32 != 0 or outfeatures % 64 != 0:
             raise ValueError("`infeatures` must be divisible by 32 and `outfeatures` by 64.")
+        if out_dtype not in (None, torch.float16, torch.float32):
+            raise ValueError("out_dtype must be None, torch.float16 or torch.float32")
         self.infeatures = infeatures
         self.outfeatures = outfeatures
+        self.out_dtype = out_dtype
         self.register_buffer("packed_binary_sparse", torch.zeros((infeatures // 2, outfeatures // 8), dtype=torch.uint8))
         self.register_buffer("meta", torch.zeros((outfeatures, infeatures // 16), dtype=torch.int16))
         self.vaild = False
@@ -168,9 +176,13 @@ class BinaryLinear_2_4(nn.Module):
         self.vaild = True
         self._prepared = None
 
-    def _load_from_state_dict(self, *args, **kwargs):
-        super()._load_from_state_dict(*args, **kwargs)
-        self.vaild = True
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                              error_msgs):
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                                      error_msgs)
+        # a packed weight is there only if both buffers came from the state dict
+        if prefix + "packed_binary_sparse" in state_dict and prefix + "meta" in state_dict:
+            self.vaild = True
         self._prepared = None
 
     def forward(self, x):
@@ -185,6 +197,8 @@ class BinaryLinear_2_4(nn.Module):
         bias = self.bias
         if bias is not None and (bias.dtype not in (torch.float16, torch.float32) or bias.device != x.device):
             bias = bias.to(device=x.device, dtype=torch.float32)
+        out_dtype = self.out_dtype or (torch.float16 if x.dtype == torch.float16 else torch.float32)
         # one kernel: reads the tokens where they lie, adds the bias, writes (tokens, outfeatures)
-        y = self._prepared.linear(tokens, bias=bias.contiguous() if bias is not None else None)
-        return y.reshape(*lead, self.outfeatures).to(x.dtype)
+        y = self._prepared.linear(tokens, bias=bias.contiguous() if bias is not None else None, out_dtype=out_dtype)
+        y = y.reshape(*lead, self.outfeatures)
+        return y if self.out_dtype is not None else y.to(x.dtype)

@@ -15,7 +15,7 @@ META_REFERENCE, META_CUTLASS, META_LOGICAL = 0, 1, 2
 EXPORTS = (
     "onebit_sparse_matmul", "onebit_sparse_matmul_ex", "onebit_sparse_prepared_bytes", "onebit_sparse_prepare",
     "onebit_sparse_matmul_prepared", "onebit_sparse_matmul_prepared_static", "onebit_sparse_linear_prepared", "onebit_sparse_pack", "onebit_sparse_last_error", "onebit_sparse_set_tile_config",
-    "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_set_split_k", "onebit_sparse_set_pad_b", "onebit_sparse_describe_launch", "onebit_sparse_set_weight_cache", "onebit_sparse_clear_weight_cache",
+    "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_set_split_k", "onebit_sparse_set_pad_b", "onebit_sparse_describe_launch", "onebit_sparse_set_weight_cache", "onebit_sparse_clear_weight_cache", "onebit_sparse_release_buffers",
     "onebit_sparse_measure_smfmac_rate", "onebit_sparse_device_info",
 )
 
@@ -61,6 +61,8 @@ def lib():
         L.onebit_sparse_set_weight_cache.argtypes = [i32]
         L.onebit_sparse_clear_weight_cache.restype = i32
         L.onebit_sparse_clear_weight_cache.argtypes = []
+        L.onebit_sparse_release_buffers.restype = i32
+        L.onebit_sparse_release_buffers.argtypes = []
         L.onebit_sparse_describe_launch.restype = i32
         L.onebit_sparse_describe_launch.argtypes = [i32, i32, i32, i32, ctypes.POINTER(ctypes.c_int)]
         L.onebit_sparse_device_info.restype = i32
@@ -183,10 +185,23 @@ def linear_prepared(prepared, x, y, m, k, bias=None):
     return y
 
 
+def _check_stored_operands(a, meta, c, d, m, n, k):
+    """Sizes of the reference-format operands: a wrong-sized tensor would be read or written out of bounds."""
+    if m % 64 or k % 32 or m <= 0 or k <= 0 or n <= 0:
+        raise ValueError("m must be a positive multiple of 64, k of 32, n positive")
+    if a.dtype != torch.uint8 or a.numel() != m * k // 16:
+        raise ValueError(f"A must be uint8 with m*k/16 = {m * k // 16} bytes (one bit per kept value)")
+    if meta.dtype != torch.int16 or meta.numel() != m * k // 16:
+        raise ValueError(f"meta must be int16 with m*k/16 = {m * k // 16} elements")
+    if tuple(d.shape) != (m, n) or (c is not None and tuple(c.shape) != (m, n)):
+        raise ValueError("C / D must have shape (m, n)")
+
+
 def matmul_ex(a, b, meta, d, m, n, k, c=None, alpha=1.0, beta=0.0, layout=META_REFERENCE):
     dev = _require_cuda(a, b, meta, d, c)
     if b.dtype != torch.float16 or tuple(b.shape) != (k, n):
         raise ValueError("B must be float16 of shape (k, n)")
+    _check_stored_operands(a, meta, c, d, m, n, k)
     with _on_device(dev):
         _check(lib().onebit_sparse_matmul_ex(
             a.data_ptr(), b.data_ptr(), c.data_ptr() if c is not None else None, d.data_ptr(), meta.data_ptr(), m, n,
@@ -197,6 +212,11 @@ def matmul_ex(a, b, meta, d, m, n, k, c=None, alpha=1.0, beta=0.0, layout=META_R
 def matmul_legacy(a, b, c, d, meta, m, n, k):
     """The 8-argument entry point: fp32 C/D, alpha = 1, beta = 0, default stream."""
     dev = _require_cuda(a, b, c, d, meta)
+    if b.dtype != torch.float16 or tuple(b.shape) != (k, n):
+        raise ValueError("B must be float16 of shape (k, n)")
+    _check_stored_operands(a, meta, c, d, m, n, k)
+    if d.dtype != torch.float32 or c.dtype != torch.float32:
+        raise TypeError("the 8-argument entry point takes float32 C and D")
     with _on_device(dev):
         lib().onebit_sparse_matmul(a.data_ptr(), b.data_ptr(), c.data_ptr(), d.data_ptr(), meta.data_ptr(), m, n, k)
     return d
@@ -264,6 +284,11 @@ def describe_launch(m, n, k, b_aligned=True):
 def set_weight_cache(entries):
     """Opt-in cache of reordered weights for the one-call entry points (0 = off, the default)."""
     _check(lib().onebit_sparse_set_weight_cache(entries))
+
+
+def release_buffers():
+    """Free the library-owned buffers of the one-call / K-split / padded-B paths (after a device synchronization)."""
+    _check(lib().onebit_sparse_release_buffers())
 
 
 def clear_weight_cache():

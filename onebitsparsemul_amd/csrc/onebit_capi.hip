@@ -5,6 +5,7 @@
 #include "onebit_device.h"
 #include "onebit_launch.h"
 
+#include <algorithm>
 #include <atomic>
 #include <cstdarg>
 #include <cstdio>
@@ -17,11 +18,13 @@
 namespace {
 
 thread_local std::string g_last_error;
-std::atomic<int> g_tile_config{-1};
-std::atomic<int> g_skinny_enabled{1};
-std::atomic<int> g_skinny_rows{-1};
-std::atomic<int> g_split_k{-1};
-std::atomic<int> g_pad_b{1};
+// Tuning / test hooks: per calling thread, so that a test or a tuning run never changes what other threads of the
+// process launch.
+thread_local int g_tile_config = -1;
+thread_local int g_skinny_enabled = 1;
+thread_local int g_skinny_rows = -1;
+thread_local int g_split_k = -1;
+thread_local int g_pad_b = 1;
 std::atomic<int> g_weight_cache_entries{0};
 
 int fail(int code, const char* fmt, ...) {
@@ -57,7 +60,8 @@ struct Buffer {
   size_t bytes = 0;
 };
 struct DeviceState {
-  std::mutex mu;
+  // recursive: the one-call entry points keep it while they launch, and the launch takes it again for its own buffers
+  std::recursive_mutex mu;
   // the reordered operand of the one-call entry points (when the weight cache is off)
   std::map<hipStream_t, Buffer> prep;
   // fp32 partial sums of the K-split passes: one buffer per stream, so that calls on different streams do not
@@ -77,6 +81,8 @@ struct DeviceState {
   };
   std::vector<CachedWeight> weight_cache;
   unsigned long use_counter = 0;
+  // compute units of the device (0 until first asked): the launch plans scale with it
+  std::atomic<int> compute_units{0};
   // this device's address of g_static_scratch (null until the first non-allocating call on the device)
   unsigned char* static_scratch = nullptr;
 };
@@ -105,6 +111,18 @@ int grow(void** ptr, size_t* have, size_t need, hipStream_t stream) {
   ONEBIT_HIP(hipMalloc(ptr, bytes));
   *have = bytes;
   return ONEBIT_OK;
+}
+
+// Compute units of the current device, asked once per device. A failure leaves the MI355X figure the plans were
+// measured on.
+int current_compute_units() {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return 256;
+  int cus = g_dev[device].compute_units.load(std::memory_order_relaxed);
+  if (cus > 0) return cus;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) cus = 256;
+  g_dev[device].compute_units.store(cus, std::memory_order_relaxed);
+  return cus;
 }
 
 int check_shape(int m, int n, int k) {
@@ -143,7 +161,7 @@ struct GemmPlan {
 
 struct TileCost {
   int tile, bm, bn;
-  int slots;        // workgroups resident on the GPU at once (256 CUs: the model is for MI355X, like the kernels)
+  int slots;        // workgroups resident at once on the 256 compute units the timings were taken on
   double chunk_us;  // K loop of one workgroup per 256-wide chunk with every slot taken
   double round_us;  // per round on top of the K loop
   bool may_split;
@@ -155,11 +173,14 @@ const TileCost kTileCosts[] = {
     {onebit::kTile64x128, 64, 128, 256, 1.0, 0.0, true},      {onebit::kTile64x128k2, 64, 128, 256, 0.88, 1.0, true},
 };
 
-double model_us(const TileCost& t, int m, int n, int chunks, int s) {
+// compute_units: of the device the call runs on. The per-chunk times are per workgroup and do not depend on it; the
+// number of resident workgroups scales with it (a partitioned or smaller GPU runs more rounds of the same tiles).
+double model_us(const TileCost& t, int m, int n, int chunks, int s, int compute_units) {
   const long tiles = (long)((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn) * s;
   const int per_split = (chunks + s - 1) / s;
-  const long full_rounds = tiles / t.slots;
-  const double f = (double)(tiles % t.slots) / t.slots;
+  const long slots = std::max(1L, (long)t.slots * compute_units / 256);
+  const long full_rounds = tiles / slots;
+  const double f = (double)(tiles % slots) / slots;
   double rounds = (double)full_rounds;
   if (f > 0.0) rounds += t.slots == 256 ? (f > 0.9 ? 1.0 : 0.85) : (f <= 0.5 ? 0.6 : 1.0);
   double us = 4.0 + (t.chunk_us * per_split + t.round_us) * rounds;
@@ -167,10 +188,10 @@ double model_us(const TileCost& t, int m, int n, int chunks, int s) {
   return us;
 }
 
-GemmPlan plan_gemm(int m, int n, int k) {
+GemmPlan plan_gemm(int m, int n, int k, int compute_units) {
   const int chunks = (k + onebit::kChunkK - 1) / onebit::kChunkK;
-  const int forced_tile = g_tile_config.load();
-  const int forced_splits = g_split_k.load();
+  const int forced_tile = g_tile_config;
+  const int forced_splits = g_split_k;
   if (forced_tile >= 0) {
     // a forced tile of the table may still be split by the model
     int splits = forced_splits >= 1 ? forced_splits : 1;
@@ -180,7 +201,7 @@ GemmPlan plan_gemm(int m, int n, int k) {
           double best_us = 1e30;
           for (int s : {1, 2, 3, 4, 6, 8, 12, 16}) {
             if (s > chunks) break;
-            const double us = model_us(t, m, n, chunks, s);
+            const double us = model_us(t, m, n, chunks, s, compute_units);
             if (us < best_us) best_us = us, splits = s;
           }
         }
@@ -191,7 +212,7 @@ GemmPlan plan_gemm(int m, int n, int k) {
   GemmPlan best{onebit::kTile128x128s, fixed_splits ? fixed_splits : 1};
   double best_us = 1e30;
   auto consider = [&](const TileCost& t, int s) {
-    const double us = model_us(t, m, n, chunks, s);
+    const double us = model_us(t, m, n, chunks, s, compute_units);
     if (us < best_us) {
       best_us = us;
       best = GemmPlan{t.tile, s};
@@ -218,30 +239,31 @@ struct LaunchPlan {
   int pad_b;           // gemm_kernel: B is read through a padded copy
 };
 
-LaunchPlan choose_launch(int m, int n, int k, bool b_16_byte_aligned) {
+LaunchPlan choose_launch(int m, int n, int k, bool b_16_byte_aligned, int compute_units = 256) {
   LaunchPlan plan{};
   // 32 < n <= 64: every 64-row workgroup of the split-K kernel stages all of B, which the main kernel's tiles overtake
   // from about 48k rows on (n = 64: 28672 x 8192 32 us against 42; 32768 x 4096 20 against 26; 49152 x 4096 32.5
   // against 34.4; 65536 x 8192 66 against 68, at n = 40 77 against 66; 131072 x 2048 51 against 35)
   const bool skinny_shape = n <= 32 || (n <= onebit::kSkinnyMaxN && m <= 40960);
-  if (skinny_shape && g_skinny_enabled.load()) {
-    int rows = g_skinny_rows.load();
+  if (skinny_shape && g_skinny_enabled) {
+    int rows = g_skinny_rows;
     // the largest row group that still gives about two workgroups per three compute units (measured: larger groups
     // re-read B less often, but idle compute units cost more)
     // (n > 32: two column fragments per row block, at most two row blocks per wavefront)
-    if (rows <= 0) rows = (m / 128 >= 160 && n <= 32) ? 128 : (m / 64 >= 160) ? 64 : 32;
+    const int enough = std::max(1, 160 * compute_units / 256);  // about two workgroups per three compute units
+    if (rows <= 0) rows = (m / 128 >= enough && n <= 32) ? 128 : (m / 64 >= enough) ? 64 : 32;
     plan.split_k_kernel = 1;
     plan.rows_or_tile = rows;
     plan.splits = 1;
     return plan;
   }
-  const GemmPlan gemm = plan_gemm(m, n, k);
+  const GemmPlan gemm = plan_gemm(m, n, k, compute_units);
   plan.rows_or_tile = gemm.tile;
   plan.splits = gemm.splits;
   // B rows that are not 16-byte aligned: pad a copy (one extra pass over B) unless the problem is too small for that
   // to pay against the element-copy variant of the kernel
   const bool b_in_place = n % 8 == 0 && b_16_byte_aligned;
-  plan.pad_b = !b_in_place && (size_t)k * n >= 65536 && g_pad_b.load();
+  plan.pad_b = !b_in_place && (size_t)k * n >= 65536 && g_pad_b;
   return plan;
 }
 
@@ -258,7 +280,7 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
   if (beta != 0.f && !c) return fail(ONEBIT_ERR_ARGUMENT, "c must not be null when beta != 0");
   const int kc_total = (k + onebit::kChunkK - 1) / onebit::kChunkK;
 
-  const LaunchPlan plan = choose_launch(m, n, k, (reinterpret_cast<uintptr_t>(b) & 15) == 0);
+  const LaunchPlan plan = choose_launch(m, n, k, (reinterpret_cast<uintptr_t>(b) & 15) == 0, current_compute_units());
   if (plan.split_k_kernel) {
     onebit::SkinnyArgs args{};
     args.prep = static_cast<const uint8_t*>(prepared);
@@ -274,6 +296,10 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
     return ONEBIT_OK;
   }
 
+  if (onebit::prepared_bytes(m, k) >= (size_t(1) << 32))
+    return fail(ONEBIT_ERR_ARGUMENT,
+                "the main kernel addresses the prepared operand with 32-bit offsets: m x k = %d x %d needs %zu bytes, "
+                "the limit is 4 GiB (about 22.9e9 weights); split the weight by rows", m, k, onebit::prepared_bytes(m, k));
   onebit::GemmArgs args{};
   args.prep = static_cast<const uint8_t*>(prepared);
   args.b = static_cast<const _Float16*>(b);
@@ -314,7 +340,7 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
     ONEBIT_HIP(hipGetDevice(&device));
     if (device < 0 || device >= kMaxDevices) return fail(ONEBIT_ERR_ARGUMENT, "device ordinal %d not supported", device);
     DeviceState& st = g_dev[device];
-    std::lock_guard<std::mutex> lock(st.mu);
+    std::lock_guard<std::recursive_mutex> lock(st.mu);
     if (splits > 1) {
       Buffer& ws = st.split_ws[stream];
       if (int rc = grow(&ws.ptr, &ws.bytes, split_bytes, stream); rc != ONEBIT_OK) return rc;
@@ -338,11 +364,11 @@ extern "C" {
 
 const char* onebit_sparse_last_error(void) { return g_last_error.c_str(); }
 
-void onebit_sparse_set_tile_config(int tile_config) { g_tile_config.store(tile_config); }
-void onebit_sparse_set_skinny_enabled(int enabled) { g_skinny_enabled.store(enabled ? 1 : 0); }
-void onebit_sparse_set_skinny_rows(int rows) { g_skinny_rows.store(rows); }
-void onebit_sparse_set_split_k(int splits) { g_split_k.store(splits); }
-void onebit_sparse_set_pad_b(int enabled) { g_pad_b.store(enabled ? 1 : 0); }
+void onebit_sparse_set_tile_config(int tile_config) { g_tile_config = tile_config; }
+void onebit_sparse_set_skinny_enabled(int enabled) { g_skinny_enabled = enabled ? 1 : 0; }
+void onebit_sparse_set_skinny_rows(int rows) { g_skinny_rows = rows; }
+void onebit_sparse_set_split_k(int splits) { g_split_k = splits; }
+void onebit_sparse_set_pad_b(int enabled) { g_pad_b = enabled ? 1 : 0; }
 
 int onebit_sparse_describe_launch(int m, int n, int k, int b_16_byte_aligned, int* plan) {
   g_last_error.clear();
@@ -404,7 +430,7 @@ int onebit_sparse_matmul_prepared_static(const void* prepared, const void* b, co
   DeviceState& st = g_dev[device];
   FixedScratch fixed{nullptr, kStaticScratchBytes};
   {
-    std::lock_guard<std::mutex> lock(st.mu);
+    std::lock_guard<std::recursive_mutex> lock(st.mu);
     if (!st.static_scratch) {
       // once per device, with that device current: the address of this device's copy of the array
       void* address = nullptr;
@@ -426,7 +452,10 @@ int onebit_sparse_linear_prepared(const void* prepared, const void* x, const voi
   if (!prepared || !x || !y) return fail(ONEBIT_ERR_ARGUMENT, "null operand pointer");
   if ((reinterpret_cast<uintptr_t>(x) & 15) != 0) return fail(ONEBIT_ERR_ARGUMENT, "x must be 16-byte aligned");
   const int kc_total = (k + onebit::kChunkK - 1) / onebit::kChunkK;
-  const LaunchPlan plan = choose_launch(m, tokens, k, true);
+  const LaunchPlan plan = choose_launch(m, tokens, k, true, current_compute_units());
+  if ((size_t)k * 256 * 2 >= (size_t(1) << 32))
+    return fail(ONEBIT_ERR_ARGUMENT, "the token-major form addresses x with 32-bit offsets inside a tile of 256 tokens: "
+                                     "k = %d is beyond its limit of 8388607", k);
   if (plan.split_k_kernel) {
     onebit::SkinnyArgs args{};
     args.prep = static_cast<const uint8_t*>(prepared);
@@ -448,6 +477,10 @@ int onebit_sparse_linear_prepared(const void* prepared, const void* x, const voi
       return fail(ONEBIT_ERR_ARGUMENT, "tile configuration %d has no token-major variant (4, 6, 9 ... 14 have)",
                   plan.rows_or_tile);
   }
+  if (onebit::prepared_bytes(m, k) >= (size_t(1) << 32))
+    return fail(ONEBIT_ERR_ARGUMENT,
+                "the main kernel addresses the prepared operand with 32-bit offsets: m x k = %d x %d needs %zu bytes, "
+                "the limit is 4 GiB (about 22.9e9 weights); split the weight by rows", m, k, onebit::prepared_bytes(m, k));
   onebit::GemmArgs args{};
   args.prep = static_cast<const uint8_t*>(prepared);
   args.b = static_cast<const _Float16*>(x);
@@ -463,7 +496,7 @@ int onebit_sparse_linear_prepared(const void* prepared, const void* x, const voi
     ONEBIT_HIP(hipGetDevice(&device));
     if (device < 0 || device >= kMaxDevices) return fail(ONEBIT_ERR_ARGUMENT, "device ordinal %d not supported", device);
     DeviceState& st = g_dev[device];
-    std::lock_guard<std::mutex> lock(st.mu);
+    std::lock_guard<std::recursive_mutex> lock(st.mu);
     const int cps = (kc_total + plan.splits - 1) / plan.splits;
     args.chunks_per_split = cps;
     args.splits = (kc_total + cps - 1) / cps;  // every split non-empty
@@ -495,7 +528,7 @@ int onebit_sparse_matmul_ex(const void* a, const void* b, const void* c, void* d
   const int cache_entries = g_weight_cache_entries.load();
   if (cache_entries > 0) {
     {  // the lock ends before the multiplication is launched, which may take it again for its own buffers
-      std::lock_guard<std::mutex> lock(ds.mu);
+      std::lock_guard<std::recursive_mutex> lock(ds.mu);
       for (auto& w : ds.weight_cache)
         if (w.a == a && w.e == e && w.m == m && w.k == k && w.layout == meta_layout) {
           w.last_use = ++ds.use_counter;
@@ -537,12 +570,12 @@ int onebit_sparse_matmul_ex(const void* a, const void* b, const void* c, void* d
     }
     return matmul_prepared_impl(prep, b, c, d, m, n, k, alpha, beta, c_dtype, d_dtype, s);
   }
-  {
-    std::lock_guard<std::mutex> lock(ds.mu);
-    Buffer& own = ds.prep[s];
-    if (int rc = grow(&own.ptr, &own.bytes, onebit::prepared_bytes(m, k), s)) return rc;
-    prep = own.ptr;
-  }
+  // the lock is kept until both kernels are enqueued: a call from another thread that has to grow this stream's
+  // buffer (which frees the old one) then waits, and its device synchronization covers the work enqueued here
+  std::lock_guard<std::recursive_mutex> lock(ds.mu);
+  Buffer& own = ds.prep[s];
+  if (int rc = grow(&own.ptr, &own.bytes, onebit::prepared_bytes(m, k), s)) return rc;
+  prep = own.ptr;
   ONEBIT_HIP(onebit::launch_prepare(a, e, prep, m, k, meta_layout, s));
   return matmul_prepared_impl(prep, b, c, d, m, n, k, alpha, beta, c_dtype, d_dtype, s);
 }
@@ -554,7 +587,7 @@ int onebit_sparse_clear_weight_cache(void) {
   int rc = ONEBIT_OK;
   for (int device = 0; device < kMaxDevices; ++device) {
     DeviceState& ds = g_dev[device];
-    std::lock_guard<std::mutex> lock(ds.mu);
+    std::lock_guard<std::recursive_mutex> lock(ds.mu);
     if (ds.weight_cache.empty()) continue;
     if (hipSetDevice(device) != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
       rc = fail(ONEBIT_ERR_HIP, "cannot synchronize device %d to clear its weight cache", device);
@@ -565,6 +598,29 @@ int onebit_sparse_clear_weight_cache(void) {
       (void)hipEventDestroy(w.ready);
     }
     ds.weight_cache.clear();
+  }
+  if (have_device) (void)hipSetDevice(previous);
+  return rc;
+}
+
+int onebit_sparse_release_buffers(void) {
+  g_last_error.clear();
+  int previous = 0;
+  const bool have_device = hipGetDevice(&previous) == hipSuccess;
+  int rc = ONEBIT_OK;
+  for (int device = 0; device < kMaxDevices; ++device) {
+    DeviceState& ds = g_dev[device];
+    std::lock_guard<std::recursive_mutex> lock(ds.mu);
+    if (ds.prep.empty() && ds.split_ws.empty() && ds.b_pad.empty()) continue;
+    if (hipSetDevice(device) != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
+      rc = fail(ONEBIT_ERR_HIP, "cannot synchronize device %d to release its buffers", device);
+      continue;
+    }
+    for (auto* buffers : {&ds.prep, &ds.split_ws, &ds.b_pad}) {
+      for (auto& entry : *buffers)
+        if (entry.second.ptr) (void)hipFree(entry.second.ptr);
+      buffers->clear();
+    }
   }
   if (have_device) (void)hipSetDevice(previous);
   return rc;

@@ -259,54 +259,11 @@ __device__ __forceinline__ void compute_stage(const char* stage_lds, const AChun
   }
 }
 
-// Compile-time experiment switches (all off in the shipped build): each removes one ingredient of the main
-// loop so that its cost can be measured; results are wrong when any of them is set.
-#ifndef ONEBIT_EXP_NO_LDS_READ
-#define ONEBIT_EXP_NO_LDS_READ 0
-#endif
-#ifndef ONEBIT_EXP_NO_EXPAND
-#define ONEBIT_EXP_NO_EXPAND 0
-#endif
-#ifndef ONEBIT_EXP_NO_COPY
-#define ONEBIT_EXP_NO_COPY 0
-#endif
-#ifndef ONEBIT_EXP_COPY_MODE  /* 1: no A copies, 2: no B copies, 3: B copies never advance (always cache hits),
-                                 5: only every other B copy (half the L2->LDS traffic, same addresses otherwise) */
-#define ONEBIT_EXP_COPY_MODE 0
-#endif
-#ifndef ONEBIT_EXP_WAIT_MODE  /* 1: never wait for copies (vmcnt 63), 2: always wait for all copies (vmcnt 0) */
-#define ONEBIT_EXP_WAIT_MODE 0
-#endif
-#ifndef ONEBIT_MAIN_ORDER    /* SMFMAC order inside a K step: 0 row fragments outer (A held), 1 column fragments outer (B held) */
-#define ONEBIT_MAIN_ORDER 0
-#endif
-#ifndef ONEBIT_MAIN_PINNED   /* 1: inline-asm SMFMAC with accumulators pinned to AGPRs where that fits, 0: builtin */
-#define ONEBIT_MAIN_PINNED 1
-#endif
-#ifndef ONEBIT_MAIN_INTERLEAVE /* 1: force the order SMFMAC, LDS read, VALU inside each K-step region */
-#define ONEBIT_MAIN_INTERLEAVE 0
-#endif
-#ifndef ONEBIT_EXP_EXTRA  /* marginal-cost probes, data unchanged: 1: every sign expansion is computed twice,
-                             2: every transpose read is issued twice, 3: every B copy is issued twice */
-#define ONEBIT_EXP_EXTRA 0
-#endif
-#ifndef ONEBIT_EXP_NO_BARRIER
-#define ONEBIT_EXP_NO_BARRIER 0
-#endif
-#ifndef ONEBIT_EXP_NO_STORE
-#define ONEBIT_EXP_NO_STORE 0
-#endif
-
 // ---- software-pipelined building blocks of the asynchronous-copy main loop -------------------------
 // B fragments of one 32-wide K step (ks = 0/1 inside a 64-row stage image).
 template <int FN, int BN>
 __device__ __forceinline__ void load_b_frags(const char* stage_lds, int ks, half16_t (&bv)[FN], const int (&frag_off)[FN],
                                              int lane_row_off) {
-  if (ONEBIT_EXP_NO_LDS_READ) {
-#pragma unroll
-    for (int fn = 0; fn < FN; ++fn) asm volatile("" : "+v"(bv[fn]));
-    return;
-  }
 #pragma unroll
   for (int fn = 0; fn < FN; ++fn) {
     u32x8_t raw;
@@ -316,12 +273,6 @@ __device__ __forceinline__ void load_b_frags(const char* stage_lds, int ks, half
       const u32x2_t t = lds_read_tr16(stage_lds + lane_row_off + row_const * (BN * 2) + frag_off[fn]);
       raw[2 * q] = t.x;
       raw[2 * q + 1] = t.y;
-      if (ONEBIT_EXP_EXTRA == 2) {
-        int again = lane_row_off;
-        asm volatile("" : "+v"(again));
-        const u32x2_t t2 = lds_read_tr16(stage_lds + again + row_const * (BN * 2) + frag_off[fn]);
-        asm volatile("" ::"v"(t2));
-      }
     }
     bv[fn] = __builtin_bit_cast(half16_t, raw);
   }
@@ -355,21 +306,8 @@ __device__ __forceinline__ void load_b_frags_tokens(const char* wave_lds, int ks
 
 template <int STEP, int FM>
 __device__ __forceinline__ void expand_frags(const AChunk (&a)[FM], uint32_t one, half8_t (&av)[FM]) {
-  if (ONEBIT_EXP_NO_EXPAND) {
 #pragma unroll
-    for (int fm = 0; fm < FM; ++fm) asm volatile("" : "+v"(av[fm]));
-    return;
-  }
-#pragma unroll
-  for (int fm = 0; fm < FM; ++fm) {
-    av[fm] = expand_signs<STEP>(a[fm], one);
-    if (ONEBIT_EXP_EXTRA == 1) {
-      AChunk again = a[fm];
-      asm volatile("" : "+v"(again.sign));
-      const half8_t av2 = expand_signs<STEP>(again, one);
-      asm volatile("" ::"v"(av2));
-    }
-  }
+  for (int fm = 0; fm < FM; ++fm) av[fm] = expand_signs<STEP>(a[fm], one);
 }
 
 template <int STEP, int FM, int FN>
@@ -377,39 +315,10 @@ __device__ __forceinline__ void mfma_frags(const AChunk (&a)[FM], const half8_t 
                                            float16_t (&acc)[FM][FN]) {
   // pinned accumulators only for the one-wavefront-per-SIMD tiles: the two-per-SIMD tiles have 128 vector
   // registers left beside their 128 accumulators, which the pinned form overflows
-#if ONEBIT_MAIN_ORDER == 1
-#pragma unroll
-  for (int fn = 0; fn < FN; ++fn)
-#pragma unroll
-    for (int fm = 0; fm < FM; ++fm)
-      acc[fm][fn] = smfmac_step<STEP, (ONEBIT_MAIN_PINNED != 0 && FM * FN > 8)>(a[fm], av[fm], bv[fn], acc[fm][fn]);
-#else
 #pragma unroll
   for (int fm = 0; fm < FM; ++fm)
 #pragma unroll
-    for (int fn = 0; fn < FN; ++fn)
-      acc[fm][fn] = smfmac_step<STEP, (ONEBIT_MAIN_PINNED != 0 && FM * FN > 8)>(a[fm], av[fm], bv[fn], acc[fm][fn]);
-#endif
-}
-
-// Pins the instruction order of one K-step region: each SMFMAC is followed by its share of the region's LDS
-// reads (4 FN in total) and sign-expansion VALU instructions (8 FM in total).
-template <int FM, int FN, int I>
-__device__ __forceinline__ void interleave_from() {
-  if constexpr (I < FM * FN) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    constexpr int DS = (4 * FN * (I + 1)) / (FM * FN) - (4 * FN * I) / (FM * FN);
-    constexpr int VA = (8 * FM * (I + 1)) / (FM * FN) - (8 * FM * I) / (FM * FN);
-    if constexpr (DS > 0) __builtin_amdgcn_sched_group_barrier(0x100, DS, 0);
-    if constexpr (VA > 0) __builtin_amdgcn_sched_group_barrier(0x002, VA, 0);
-    interleave_from<FM, FN, I + 1>();
-  }
-}
-template <int FM, int FN>
-__device__ __forceinline__ void interleave_region() {
-#if ONEBIT_MAIN_INTERLEAVE
-  interleave_from<FM, FN, 0>();
-#endif
+    for (int fn = 0; fn < FN; ++fn) acc[fm][fn] = smfmac_step<STEP, (FM * FN > 8)>(a[fm], av[fm], bv[fn], acc[fm][fn]);
 }
 
 // Source of zeros for the asynchronous copies of B rows at or past K.
@@ -530,14 +439,9 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
     // whole chunks of four stages) and the padding of the prepared operand contribute nothing, and the
     // number of copies in flight, which the vmcnt waits rely on, is the same in every iteration.
     auto issue_b = [&](int ring) {
-      if (ONEBIT_EXP_NO_COPY || ONEBIT_EXP_COPY_MODE == 2) return;
       if (next_k0 + kStageK <= p.k) {  // wave-uniform: a full stage
 #pragma unroll
-        for (int i = 0; i < NL; ++i)
-          if (ONEBIT_EXP_COPY_MODE != 5 || (i & 1) == 0) {
-            lds_dma16_base(b_stage, b_off[i], lds_dst[i] + ring * TS::STAGE_BYTES);
-            if (ONEBIT_EXP_EXTRA == 3) lds_dma16_base(b_stage, b_off[i], lds_dst[i] + ring * TS::STAGE_BYTES);
-          }
+        for (int i = 0; i < NL; ++i) lds_dma16_base(b_stage, b_off[i], lds_dst[i] + ring * TS::STAGE_BYTES);
       } else {
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
@@ -545,7 +449,7 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
           lds_dma16(src, lds_dst[i] + ring * TS::STAGE_BYTES);
         }
       }
-      if (ONEBIT_EXP_COPY_MODE != 3) b_stage += stage_stride;
+      b_stage += stage_stride;
       next_k0 += kStageK;
     };
 
@@ -572,7 +476,6 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
     const char* a_chunk = reinterpret_cast<const char*>(p.prep) + (size_t)chunk_begin * kBlockBytes;  // advances one K chunk per copy
     int next_chunk = chunk_begin;
     auto issue_a = [&]() {
-      if (ONEBIT_EXP_NO_COPY || ONEBIT_EXP_COPY_MODE == 1) return;
 #pragma unroll
       for (int j = 0; j < NA; ++j) lds_dma16_base(a_chunk, a_off[j], a_dst[j]);
       if (next_chunk + 1 < chunks) a_chunk += kBlockBytes;  // past the last chunk the last one is copied again
@@ -608,10 +511,9 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
         read_frags((S), 1, bv1);                                                                                   \
         expand_frags<2 * (S) + 1>(a_cur, one, av1);                                                                \
         mfma_frags<2 * (S)>(a_cur, av0, bv0, acc);                                                                 \
-        interleave_region<FM, FN>();                                                                               \
         __builtin_amdgcn_sched_barrier(0); /* keep the step's work inside its region */                           \
-        wait_vmcnt_lgkm0<(ONEBIT_EXP_WAIT_MODE == 1 ? 63 : ONEBIT_EXP_WAIT_MODE == 2 ? 0 : (WAITCNT))>(); /* copies of stage S+1 landed; this wavefront's reads of stage S returned */ \
-        if (!ONEBIT_EXP_NO_BARRIER) __builtin_amdgcn_s_barrier();                                                  \
+        wait_vmcnt_lgkm0<(WAITCNT)>(); /* copies of stage S+1 landed; this wavefront's reads of stage S returned */      \
+        __builtin_amdgcn_s_barrier();                                                                              \
         if (ISSUE_A) issue_a();                                                                                    \
         issue_b(S);                                                                                                \
         read_frags(((S) + 1) % kStages, 0, bv0);                                                                   \
@@ -622,19 +524,16 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
         ONEBIT_STAGE(0, 2 * NL, true)
         expand_frags<2>(a_cur, one, av0);
         mfma_frags<1>(a_cur, av1, bv1, acc);
-        interleave_region<FM, FN>();
         __builtin_amdgcn_sched_barrier(0);
         // mid stage 1: waits for B(4c+2); newer: B(4c+3), A(c+1), B(4c+4)
         ONEBIT_STAGE(1, 2 * NL + NA, false)
         expand_frags<4>(a_cur, one, av0);
         mfma_frags<3>(a_cur, av1, bv1, acc);
-        interleave_region<FM, FN>();
         __builtin_amdgcn_sched_barrier(0);
         // mid stage 2: waits for B(4c+3); newer: A(c+1), B(4c+4), B(4c+5)
         ONEBIT_STAGE(2, 2 * NL + NA, false)
         expand_frags<6>(a_cur, one, av0);
         mfma_frags<5>(a_cur, av1, bv1, acc);
-        interleave_region<FM, FN>();
         __builtin_amdgcn_sched_barrier(0);
         // mid stage 3: waits for B(4c+4), which is newer than A(c+1): the next chunk of A is readable after it
         ONEBIT_STAGE(3, 2 * NL, false)
@@ -647,7 +546,6 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
 #pragma unroll
           for (int fm = 0; fm < FM; ++fm) a_cur[fm] = a_next[fm];
         }
-        interleave_region<FM, FN>();
         __builtin_amdgcn_sched_barrier(0);
       }
 #undef ONEBIT_STAGE
@@ -936,7 +834,7 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
             const float4 lo = *reinterpret_cast<const float4*>(scratch + r * WCOLS + c8);
             const float4 hi = *reinterpret_cast<const float4*>(scratch + r * WCOLS + c8 + 4);
             float x[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-            if (row < row_limit && col < p.n && !(ONEBIT_EXP_NO_STORE && x[0] != 12345.f)) {
+            if (row < row_limit && col < p.n) {
               const size_t o = (size_t)row * p.n + col;
 #pragma unroll
               for (int j = 0; j < 8; ++j) x[j] = p.alpha * x[j];
@@ -989,7 +887,7 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
             const int row = row_base + r, col = col0 + c4;
             const float4 a4 = *reinterpret_cast<const float4*>(scratch + r * WCOLS + c4);
             float x[4] = {a4.x, a4.y, a4.z, a4.w};
-            if (row < row_limit && col < p.n && !(ONEBIT_EXP_NO_STORE && x[0] != 12345.f)) {
+            if (row < row_limit && col < p.n) {
               const size_t o = (size_t)row * p.n + col;
 #pragma unroll
               for (int j = 0; j < 4; ++j) x[j] = p.alpha * x[j];
@@ -1023,7 +921,7 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int row = row0 + fm * 32 + 8 * (v / 4) + row_lane + (v % 4);
-        if (row < row_limit && col < p.n && !(ONEBIT_EXP_NO_STORE && acc[fm][fn][v] != 12345.f)) {
+        if (row < row_limit && col < p.n) {
           const size_t o = (size_t)row * p.n + col;
           float x = p.alpha * acc[fm][fn][v];
           if (p.beta != 0.f) {
@@ -1051,9 +949,6 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
 // (deterministic; the tiles take the place of the images, as many row blocks per round as fit the 8 KiB) and the
 // epilogue is applied. grid = M / (32 R) workgroups; no global workspace, no atomics.
 // =====================================================================================================
-#ifndef ONEBIT_EXP_SKINNY
-#define ONEBIT_EXP_SKINNY 0  // measurement builds (results wrong): 1 no B reloads, 2 one fragment group per chunk, 3 one expansion per chunk, 4 loads and image stores only
-#endif
 constexpr int kSkinnyRegion = 8192;  // bytes of one B image
 
 // how B rows reach the image: whole rows are the image rows (n == NC), rows of n % 8 == 0 elements in 16-byte
@@ -1284,20 +1179,13 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
       constexpr int STEP = decltype(step_tag)::value;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-#if ONEBIT_EXP_SKINNY == 3
-        const half8_t av = expand_signs<0>(a[0], one);
-#else
         const half8_t av = expand_signs<STEP>(a[r], one);
-#endif
 #pragma unroll
         for (int f = 0; f < NF; ++f) acc[r][f] = smfmac_step<STEP, false>(a[r], av, bfrag[STEP % FG][f], acc[r][f]);
       }
     };
     auto group = [&](auto first_tag) __attribute__((always_inline)) {
       constexpr int FIRST = decltype(first_tag)::value;  // step within the chunk
-#if ONEBIT_EXP_SKINNY == 2
-      if (FIRST == 0)
-#endif
 #pragma unroll
       for (int st = 0; st < FG; ++st)
 #pragma unroll
@@ -1349,14 +1237,8 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
     const int k_base = kc * kChunkK;
     if (!kPrefetchB) load_b(k_base, breg);
     store_b(k_base, breg);  // after the previous image's fragment reads: LDS operations of a wavefront execute in order
-#if ONEBIT_EXP_SKINNY != 1
     if (kPrefetchB) load_b(SUB > 1 ? k_base + IMG_ROWS : k_base + NW * kChunkK, breg);
-#endif
     load_a(kc + NW, a_next);
-#if ONEBIT_EXP_SKINNY == 4
-#pragma unroll
-    for (int r = 0; r < R; ++r) acc[r][0][0] += __builtin_bit_cast(float, a_cur[r].meta.x ^ a_cur[r].sign.y);
-#else
     compute(a_cur, std::integral_constant<int, 0>{});
     // the chunk's further images (SUB - 1 of them)
     auto further = [&](auto sub_tag) __attribute__((always_inline)) {
@@ -1375,7 +1257,6 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
     further(std::integral_constant<int, 1>{});
     further(std::integral_constant<int, 2>{});
     further(std::integral_constant<int, 3>{});
-#endif
 #pragma unroll
     for (int r = 0; r < R; ++r) a_cur[r] = a_next[r];
   }

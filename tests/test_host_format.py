@@ -143,3 +143,17 @@ def test_synthetic_weight_is_valid_2to4(oracle_lib):
     a2, meta2 = synthetic.make_weight(128, 64, seed=7)
     assert torch.equal(a, a2) and torch.equal(meta, meta2)
     assert set(np.unique(dense).tolist()) == {-1, 0, 1}
+
+
+def test_layer_is_valid_only_after_its_buffers_were_loaded():
+    """A state dict without the packed weight must not mark the layer as holding one (strict=False loads)."""
+    import onebitsparsemul_amd as ob
+    layer = ob.BinaryLinear_2_4(64, 64)
+    layer.load_state_dict({}, strict=False)
+    assert not layer.vaild
+    donor = ob.BinaryLinear_2_4(64, 64)
+    donor.pack(torch.randn(64, 64))
+    layer.load_state_dict(donor.state_dict())
+    assert layer.vaild and torch.equal(layer.meta, donor.meta)
+    with pytest.raises(ValueError):
+        ob.BinaryLinear_2_4(64, 64, out_dtype=torch.bfloat16)

@@ -216,3 +216,55 @@ def test_layer_forward_of_an_empty_batch():
     assert tuple(out.shape) == (0, 128) and out.dtype == torch.float16
     out = layer(torch.empty((2, 0, 64), dtype=torch.float16, device="cuda"))
     assert tuple(out.shape) == (2, 0, 128)
+
+
+def test_layer_result_dtype_follows_the_activations():
+    """float16 activations: float16 result; other activation dtypes (and out_dtype=float32): the kernel's fp32 result,
+    so sums beyond float16's range survive. Integer operands: exact against the oracle."""
+    import onebitsparsemul_amd as ob
+    in_f, out_f, tokens = 2048, 256, 9
+    a, meta = synthetic.make_weight(out_f, in_f, seed=77)
+    dense = oracle.decompress_operands(a.numpy(), meta.numpy(), out_f, in_f)
+    x = synthetic.make_b(tokens, in_f, seed=78, kind="int").float() * 256.0  # sums of 1024 terms of up to 2048: beyond 65504
+    want = _expected(dense, x.numpy(), None, np.float32)
+    assert np.abs(want).max() > 65504.0
+    for out_dtype, x_dtype, got_dtype in ((None, torch.float32, torch.float32), (None, torch.bfloat16, torch.bfloat16),
+                                          (torch.float32, torch.float16, torch.float32)):
+        layer = ob.BinaryLinear_2_4(in_f, out_f, out_dtype=out_dtype)
+        layer.packed_binary_sparse, layer.meta, layer.vaild = a, meta, True
+        layer = layer.cuda()
+        got = layer(x.to(x_dtype).cuda())
+        torch.cuda.synchronize()
+        assert got.dtype == got_dtype
+        if got_dtype == torch.float32:
+            assert np.array_equal(got.cpu().numpy(), want)
+        else:  # the fp32 sums rounded once to the activation dtype
+            assert torch.equal(got.cpu(), torch.from_numpy(want).to(got_dtype))
+    # float16 in, float16 out (the default): the same sums overflow to infinity, as a float16 result must
+    layer = ob.BinaryLinear_2_4(in_f, out_f)
+    layer.packed_binary_sparse, layer.meta, layer.vaild = a, meta, True
+    got = layer.cuda()(x.half().cuda())
+    assert got.dtype == torch.float16 and torch.equal(got.cpu(), torch.from_numpy(want).half())
+
+
+def test_one_call_entry_points_reject_wrong_sized_operands():
+    m, n, k = 128, 8, 64
+    a, meta = synthetic.make_weight(m, k, seed=1)
+    b = synthetic.make_b(k, n, seed=2, kind="int")
+    ad, md, bd = a.cuda(), meta.cuda(), b.cuda()
+    d = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    with pytest.raises(ValueError):
+        _native.matmul_ex(ad[:-1].contiguous(), bd, md, d, m, n, k)          # A too small
+    with pytest.raises(ValueError):
+        _native.matmul_ex(ad, bd, md[:, :-1].contiguous(), d, m, n, k)       # metadata too small
+    with pytest.raises(ValueError):
+        _native.matmul_ex(ad, bd, md, d[:-1], m, n, k)                       # D too small
+    with pytest.raises(ValueError):
+        _native.matmul_ex(ad, bd, md.view(torch.uint8), d, m, n, k)          # metadata of the wrong dtype
+    with pytest.raises(ValueError):
+        _native.matmul_legacy(ad, bd, d, d[:-1], md, m, n, k)
+    with pytest.raises(TypeError):
+        _native.matmul_legacy(ad, bd, d.half(), d.half(), md, m, n, k)       # the 8-argument symbol is fp32 only
+    _native.matmul_ex(ad, bd, md, d, m, n, k)
+    torch.cuda.synchronize()
+    assert np.array_equal(d.cpu().numpy(), oracle.reference_matmul(a.numpy(), b.numpy(), meta.numpy(), m, n, k, d_dtype=oracle.F32))

@@ -5,6 +5,7 @@ import pytest
 import torch
 import torch.nn as nn
 
+import oracle
 import onebitsparsemul_amd as ob
 from onebitsparsemul_amd import replace
 
@@ -85,3 +86,79 @@ def test_replaced_model_forward_matches_dense_reference():
         want = ref(x).float().cpu().numpy()
     assert np.isfinite(got).all()
     assert np.abs(got - want).max() <= 2e-2 * np.abs(want).max()  # two chained fp16 layers with fp16 rounding between
+
+
+class _TwoLayer(nn.Module):
+    def __init__(self, d_in=256, d_hidden=512, d_out=192):
+        super().__init__()
+        self.up = nn.Linear(d_in, d_hidden, bias=False)
+        self.down = nn.Linear(d_hidden, d_out, bias=True)
+
+    def forward(self, x):
+        return self.down(torch.relu(self.up(x)))
+
+
+def _oracle_weight(weight_fp16):
+    """What a replaced layer must hold, by the oracle's restatement of the reference pipeline
+    (onebit_sparse_mul/__init__.py:130-145): magnitude mask, 2:4 compression, sign quantisation, transposed bit
+    packing; returns the stored operands and their decompressed form (-1 / 0 / +1)."""
+    w = weight_fp16.float().numpy()
+    out_f, in_f = w.shape
+    sparse, meta = oracle.sparse_from_dense(w * oracle.mask_creator(w))
+    a = oracle.pack_binary(np.ascontiguousarray(oracle.binary_quant(sparse).T))
+    return a, meta, oracle.decompress_operands(a, meta, out_f, in_f)
+
+
+def _oracle_linear(dense, x_fp16, bias_fp16, acc):
+    """y = x W^T + bias through the oracle's host GEMM on the decompressed weight, fp32 (or fp64) sums, one rounding
+    to float16 at the end (what the layer returns for float16 activations)."""
+    d = oracle.host_gemm(dense, np.ascontiguousarray(x_fp16.T), d_dtype=oracle.F32, acc=acc).T.astype(np.float64)
+    if bias_fp16 is not None:
+        d = d + bias_fp16.astype(np.float64)[None, :]
+    return d
+
+
+@pytest.mark.gpu
+def test_replaced_model_matches_the_oracle_layer_by_layer():
+    """Counterpart of the reference's model script (tests/python/test_model_replace.py:22-56) with a check it does
+    not have: every replaced layer's stored operands equal the oracle's, and its GPU forward equals the oracle's host
+    GEMM on the same input - bit for bit on integer activations, within 1e-3 on N(0,1) activations."""
+    torch.manual_seed(5)
+    net = _TwoLayer().half()
+    with torch.no_grad():
+        net.down.bias.copy_(torch.randint(-3, 4, net.down.bias.shape).half())
+    expected = {name: _oracle_weight(getattr(net, name).weight.detach()) for name in ("up", "down")}
+    bias = net.down.bias.detach().numpy().copy()
+    net = net.cuda()
+    stats = replace.replace_linear_layers(net)
+    assert sorted(stats["replaced"]) == ["down", "up"]
+    for name, (a, meta, _) in expected.items():
+        layer = getattr(net, name)
+        assert np.array_equal(layer.packed_binary_sparse.cpu().numpy(), a)       # GPU packer = oracle pipeline
+        assert np.array_equal(layer.meta.cpu().numpy(), meta)
+    seen = {}
+    hooks = [getattr(net, name).register_forward_hook(
+        lambda mod, inp, out, name=name: seen.__setitem__(name, (inp[0].detach().cpu(), out.detach().cpu())))
+        for name in ("up", "down")]
+    # integer activations: every sum is an integer below 2^24, so the only rounding is the final one to float16
+    x = torch.randint(-2, 3, (3, 7, 256)).half().cuda()
+    with torch.no_grad():
+        net(x)
+    torch.cuda.synchronize()
+    for name, b in (("up", None), ("down", bias)):
+        inp, out = seen[name]
+        want = _oracle_linear(expected[name][2], inp.reshape(-1, inp.shape[-1]).numpy(), b, "f32")
+        assert np.array_equal(out.reshape(-1, out.shape[-1]).numpy(), want.astype(np.float16)), name
+    # N(0,1) activations: each layer against the oracle on the input that layer actually received
+    x = torch.randn(4, 33, 256).half().cuda()
+    with torch.no_grad():
+        y = net(x)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y).all()
+    for name, b in (("up", None), ("down", bias)):
+        inp, out = seen[name]
+        want = _oracle_linear(expected[name][2], inp.reshape(-1, inp.shape[-1]).numpy(), b, "f64")
+        got = out.reshape(-1, out.shape[-1]).double().numpy()
+        assert np.abs(got - want).max() <= 1e-3 * np.abs(want).max(), name
+    for h in hooks:
+        h.remove()
