@@ -107,7 +107,7 @@ def run_gemm(w, steps, warmup):
     kernel_s, wall_s = time_launches(fn, steps, warmup)
     # launches shorter than the host's launch interval: also time them inside a HIP graph
     graph_s = time_graph(fn, max(steps, 200)) if 2.0 * m * n * k < 2e11 else None
-    return kernel_s, wall_s, (a, meta, b, d), graph_s
+    return kernel_s, wall_s, (a, meta, b, d), graph_s, fn
 
 
 def run_decode_rotating(m, k, n, launches=2000, copies=None):
@@ -159,9 +159,11 @@ def run_layer_form(m, k, tokens, launches=1000):
                 us_plain_kernel_pretransposed=t_plain * 1e6, us_plain_kernel_with_transposes_and_bias=t_around * 1e6)
 
 
-def cpu_baseline(w, operands, budget_s=12.0):
+def cpu_baseline(w, operands, budget_s=12.0, unit="TFLOP/s"):
     """oracle (kind 'port'): decompress + dense fp32 torch.matmul on the host cores, on a row slab sized for
-    about budget_s seconds; rate in the metric's unit (dense-equivalent TFLOP/s)."""
+    about budget_s seconds; rate in the workload's unit (dense-equivalent TFLOP/s, or algorithmic GB/s for the
+    HBM-bound decode shapes). When the slab is not the whole problem the rate is that of the slab (the rows are
+    independent, so it extrapolates linearly) and `extrapolated` says so."""
     import torch
     import oracle
     a, meta, b, d = operands
@@ -179,10 +181,32 @@ def cpu_baseline(w, operands, budget_s=12.0):
     got = d[:rows].float().cpu().numpy()
     scale = float(abs(out).max())
     rel = float(abs(got - w["alpha"] * out).max() / scale) if w["beta"] == 0.0 else None
-    return dict(value=2.0 * rows * n * k / t_mm / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+    if unit == "GB/s":
+        value = algorithmic_bytes(rows, n, k, w["beta"]) / t_mm / 1e9
+    else:
+        value = 2.0 * rows * n * k / t_mm / 1e12
+    return dict(value=value, unit=unit, cores=torch.get_num_threads(), kind="port",
                 sample=f"rows 0..{rows} of {m} (all of K={k}, N={n}): decompress {t_dec:.2f}s once + fp32 torch.matmul "
-                       f"{t_mm:.2f}s each, {repeats} repetitions",
-                gpu_vs_oracle_rel_err_on_sample=rel)
+                       f"{t_mm:.4f}s each, {repeats} repetitions",
+                extrapolated=rows < m, gpu_vs_oracle_rel_err_on_sample=rel)
+
+
+def sustained_rate(fn, flops, load_ms=150.0, launches=60):
+    """The same launch after at least load_ms of continuous load (the GPU raises its clock over the first ~50 ms),
+    timed inside a HIP graph: the rate a long-running job sees, next to `value`, which times the launches right
+    after the warm-up the command line asked for."""
+    import torch
+    t0 = time.perf_counter()
+    count = 0
+    while (time.perf_counter() - t0) * 1e3 < load_ms:
+        for _ in range(10):
+            fn(0)
+        torch.cuda.synchronize()
+        count += 10
+    t = time_graph(fn, launches, warmup=10)
+    return dict(ms_per_step=t * 1e3, tflops=flops / t / 1e12, frac=flops / t / 1e12 / SMFMAC_PEAK_TFLOPS,
+                preceding_load_ms=(time.perf_counter() - t0) * 1e3, preceding_launches=count, graph_launches=launches,
+                note="HIP-graph timing of the same kernel after >= 150 ms of back-to-back launches (sustained clock)")
 
 
 def main():
@@ -196,6 +220,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-ceiling", action="store_true")
+    ap.add_argument("--no-sustained", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one elementwise copy kernel over 256 MiB (reference point for HBM counters)")
     args = ap.parse_args()
@@ -211,10 +236,19 @@ def main():
     if w["name"].startswith("decode:"):
         dec = run_decode_rotating(m, k, n, launches=max(args.steps, 200))
         line = dict(metric="hbm_gbps_decode", value=dec["gbps_hbm"], unit="GB/s", n_gpus=1, steps=dec["launches"],
-                    warmup=50, ms_per_step=dec["us_per_launch_hbm"] * 1e-3, higher_is_better=True, scaling="weak",
-                    vs_baseline=None, dtype="f16", data="synthetic", config=dict(workload=w["name"]),
+                    warmup=20, ms_per_step=dec["us_per_launch_hbm"] * 1e-3, higher_is_better=True, scaling="weak",
+                    vs_baseline=None, dtype="f16", data="synthetic", config=dict(workload=w["name"], m=m, n=n, k=k),
                     roofline=dict(bound="hbm", achieved=dec["gbps_hbm"], peak=HBM_PEAK_GBS, unit="GB/s",
-                                  frac=dec["frac_of_hbm_peak"], traffic=None), decode=dec)
+                                  frac=dec["frac_of_hbm_peak"], traffic=MEASURED_TRAFFIC_BYTES.get(w["name"])),
+                    decode=dec)
+        if not args.no_cpu_baseline:
+            from onebitsparsemul_amd import _native, synthetic
+            a, meta = synthetic.make_weight(m, k, seed=3, device="cuda")
+            b = synthetic.make_b(k, n, seed=4, kind="normal", device="cuda")
+            d = torch.empty((m, n), dtype=torch.float16, device="cuda")
+            _native.matmul_prepared(_native.prepare(a, meta, m, k), b, d, m, n, k)
+            torch.cuda.synchronize()
+            line["cpu_baseline"] = cpu_baseline(w, (a, meta, b, d), unit="GB/s")
         print(json.dumps(line))
         return
 
@@ -225,7 +259,7 @@ def main():
         torch.neg(src, out=dst)
         torch.cuda.synchronize()
         del src, dst
-    kernel_s, wall_s, operands, graph_s = run_gemm(w, args.steps, args.warmup)
+    kernel_s, wall_s, operands, graph_s, fn = run_gemm(w, args.steps, args.warmup)
     tflops = 2.0 * m * n * k / kernel_s / 1e12
     line = dict(
         metric="dense_equiv_tflops", value=tflops, unit="TFLOP/s", n_gpus=1, steps=args.steps, warmup=args.warmup,
@@ -239,6 +273,8 @@ def main():
                            f"{DENSE_F16_PEAK_TFLOPS:.1f}); the same fraction as executed FLOPs MNK against the dense peak",
                       hbm_gbps_algorithmic=algorithmic_bytes(m, n, k, w["beta"]) / kernel_s / 1e9),
         wall_ms_per_step=wall_s * 1e3)
+    if not args.no_sustained:
+        line["sustained"] = sustained_rate(fn, 2.0 * m * n * k)
     if graph_s is not None:
         line["graph_ms_per_step"] = graph_s * 1e3  # the same launch inside a HIP graph: no host launch interval
         line["graph_tflops"] = 2.0 * m * n * k / graph_s / 1e12

@@ -11,7 +11,9 @@ import subprocess
 import numpy as np
 
 _DIR = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_DIR, "libonebit_oracle.so")
+# ONEBIT_ORACLE_LIBRARY overrides the default build, e.g. the sanitizer build `make -C oracle asan` (run the CPU
+# tests with it under LD_PRELOAD of gcc's libasan.so)
+_LIB_PATH = os.environ.get("ONEBIT_ORACLE_LIBRARY") or os.path.join(_DIR, "libonebit_oracle.so")
 
 LAYOUT_REFERENCE = 0
 LAYOUT_CUTLASS = 1
