@@ -1,0 +1,407 @@
+"""Host-side model of every global address the kernels form, checked against the buffers the C ABI hands them.
+
+The kernels' addresses depend on shapes, launch plan and pointers only, never on operand contents, so their index
+arithmetic can be restated on the CPU (numpy, one array element per lane) and every access asserted to lie inside its
+operand: the prepared weight, B (or its padded copy), C / D, the K-split partial sums. The model follows
+onebitsparsemul_amd/csrc/onebit_kernels.hip statement by statement (prepare_kernel, skinny_kernel with its five
+B staging modes, gemm_kernel's asynchronous copy pattern and epilogue ranges, splitk_reduce_kernel, pad_b_kernel) and
+takes the launch plan from the library itself (onebit_sparse_describe_launch, host-only). It covers the benchmark
+configurations and the long-K shapes with 33 to 64 columns (8192 x 28672 with n = 40, 48, 64). No GPU is touched.
+"""
+import numpy as np
+import pytest
+
+from onebitsparsemul_amd import _native
+
+BLOCK, SIGN_OFF, CHUNK_K, ROW_BLOCK, STAGE_K, STAGES = 1536, 1024, 256, 32, 64, 4
+LANE = np.arange(64, dtype=np.int64)
+
+# TileConfig code -> (WM, WN, FM, FN, KG), as in launch_gemm_pass
+TILES = {0: (4, 1, 4, 4, 1), 1: (4, 1, 2, 4, 1), 2: (4, 1, 1, 4, 1), 3: (2, 2, 4, 4, 1), 4: (2, 2, 4, 2, 1),
+         5: (2, 2, 8, 2, 1), 6: (2, 2, 2, 2, 1), 7: (2, 2, 4, 1, 1), 8: (2, 4, 4, 2, 1), 9: (4, 2, 4, 2, 1),
+         10: (4, 2, 2, 2, 1), 11: (2, 4, 2, 1, 1), 12: (2, 2, 1, 2, 1), 13: (2, 2, 2, 2, 2), 14: (2, 2, 1, 2, 2)}
+
+
+def prepared_bytes(m, k):
+    return ((m + 31) // 32) * ((k + 255) // 256) * BLOCK
+
+
+def inside(offsets, width, size, what):
+    offsets = np.asarray(offsets, dtype=np.int64)
+    assert offsets.size == 0 or (offsets.min() >= 0 and offsets.max() + width <= size), \
+        f"{what}: [{offsets.min()}, {offsets.max() + width}) outside a buffer of {size} bytes"
+
+
+def meta_offset_reference(r, c, m):
+    b0, b1, b2, b345 = r & 1, (r >> 1) & 1, (r >> 2) & 1, (r >> 3) & 7
+    return (c >> 1) * 2 * m + (r >> 6) * 128 + ((b1 << 6) | (b345 << 3) | (b0 << 2) | ((c & 1) << 1) | b2)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+def check_prepare(m, k):
+    kc_total, rb_total, ncols = (k + 255) // 256, m // 32, k // 16
+    a_bytes, e_elems = m * k // 16, m * ncols
+    i, ga = LANE & 31, LANE >> 5
+    for kc in {0, kc_total // 2, kc_total - 1}:
+        for rb in {0, rb_total // 2, rb_total - 1}:
+            for half in (0, 1):
+                j = kc * 128 + LANE + 64 * half
+                ok = j < k // 2
+                inside(((rb * ROW_BLOCK + j[ok] * m) >> 3), 4, a_bytes, "prepare: value bits")
+            r, c0 = rb * ROW_BLOCK + i, kc * 16 + ga
+            off = meta_offset_reference(r, c0, m)
+            for s in range(8):
+                c = c0 + 2 * s
+                ok = c < ncols
+                assert np.array_equal(off[ok], meta_offset_reference(r[ok], c[ok], m))  # the running offset is the closed form
+                inside(off[ok] * 2, 2, e_elems * 2, "prepare: metadata")
+                off = off + 2 * m
+            block = (rb * kc_total + kc) * BLOCK
+            inside(block + LANE * 16, 16, prepared_bytes(m, k), "prepare: block metadata")
+            inside(block + SIGN_OFF + LANE * 8, 8, prepared_bytes(m, k), "prepare: block signs")
+
+
+# ---------------------------------------------------------------------------------------------------------------
+def skinny_variant(n, rows, b_aligned=True, tokens=False):
+    nw, r = {32: (16, 1), 64: (8, 2), 128: (8, 4)}[rows]
+    nc = 64 if n > 32 else 32 if n > 16 else 16
+    if nc == 64:
+        r = min(r, 2)
+    if tokens:
+        mode = "tokens"
+    elif n == nc and b_aligned:
+        mode = "full"
+    elif nc > 16 and n % 8 == 0 and b_aligned:
+        mode = "b8"
+    elif nc == 16 and n == 8 and b_aligned:
+        mode = "b8"
+    elif nc == 16 and n == 4:
+        mode = "b4"
+    else:
+        mode = "scalar"
+    return nw, r, nc, mode
+
+
+def check_skinny(m, n, k, rows, tokens=False, b_aligned=True, d_size=2):
+    nw, R, nc, mode = skinny_variant(n, rows, b_aligned, tokens)
+    kc_total, rb_total = (k + 255) // 256, m // 32
+    img_rows = 8192 // (nc * 2)
+    sub = CHUNK_K // img_rows
+    prep_size, b_size = prepared_bytes(m, k), k * n * 2
+    grid = (rb_total + R - 1) // R
+    prefetch_b = nw <= 8 and mode != "scalar"
+    short_k = nw <= 8 and sub == 1 and mode != "scalar" and kc_total <= 2 * nw
+    b_fits = b_size < (1 << 32)
+    if tokens:
+        assert k * 64 * 2 < 0xFFFFFF00  # the launcher's check
+    for wg in sorted({0, 1, grid // 2, grid - 1} & set(range(grid))):
+        rb_first = wg * R
+        for wave in range(nw):
+            # --- prepared operand through one descriptor per row block
+            chunks = []
+            if short_k:
+                chunks += [wave, wave + nw]
+            else:
+                chunks.append(wave)
+                kc = wave
+                while kc < kc_total:
+                    chunks.append(kc + nw)
+                    kc += nw
+            for r in range(R):
+                rb = min(rb_first + r, rb_total - 1)
+                base, size = rb * kc_total * BLOCK, kc_total * BLOCK
+                assert size < (1 << 32)
+                for kc in chunks:
+                    block = min(kc, kc_total - 1) * BLOCK
+                    for off, width in ((LANE * 16, 16), (SIGN_OFF + LANE * 8, 8)):
+                        inside(block + off, width, size, "split-K kernel: prepared block inside its descriptor")
+                        inside(base + block + off, width, prep_size, "split-K kernel: prepared operand")
+            # --- B images
+            k_bases = []
+            if short_k:
+                k_bases += [wave * CHUNK_K, (wave + nw) * CHUNK_K]
+            else:
+                kc = wave
+                if prefetch_b:
+                    k_bases.append(wave * CHUNK_K)
+                while kc < kc_total:
+                    for s in range(sub):
+                        k_bases.append(kc * CHUNK_K + s * img_rows)
+                    if prefetch_b:
+                        k_bases.append(kc * CHUNK_K + nw * CHUNK_K)  # the next chunk's first image, possibly past K
+                    kc += nw
+            for k_base in k_bases:
+                rows_valid = min(max(k - k_base, 0), img_rows)
+                if mode == "tokens":
+                    # raw buffer loads: the descriptor (n * k * 2 bytes) checks the lane offset alone and returns zero
+                    # without an access when it is out of range; the scalar offset is added afterwards
+                    ppt = img_rows // 8
+                    tpi = 64 // ppt
+                    piece_lane, token_lane = LANE % ppt, LANE // ppt
+                    for i in range(8):
+                        if k_base + img_rows <= k:
+                            lane_off = (token_lane * k + 8 * piece_lane) * 2 + i * tpi * k * 2
+                            scalar_off = k_base * 2
+                        else:
+                            ins = k_base + 8 * piece_lane < k
+                            lane_off = np.where(ins, (token_lane * k + 8 * piece_lane) * 2 + k_base * 2 + i * tpi * k * 2,
+                                                0xFFFFFF00)
+                            scalar_off = 0
+                        assert lane_off.max() < (1 << 32)
+                        accessed = lane_off + 16 <= b_size
+                        assert np.array_equal(accessed, (token_lane + tpi * i < n) & (lane_off != 0xFFFFFF00))
+                        inside(lane_off[accessed] + scalar_off, 16, b_size, "split-K kernel: x rows")
+                    continue
+                q_all = LANE[None, :] + 64 * np.arange(8)[:, None]
+                if mode == "full":
+                    if b_fits and k_base + img_rows <= k:
+                        inside(k_base * nc * 2 + LANE[None, :] * 16 + 1024 * np.arange(8)[:, None], 16, b_size,
+                               "split-K kernel: whole B image")
+                    else:
+                        ppr = nc // 8
+                        ok = (q_all // ppr) < rows_valid
+                        inside((k_base * nc + q_all[ok] * 8) * 2, 16, b_size, "split-K kernel: B image pieces")
+                elif mode == "b8":
+                    ppr = nc // 8
+                    row, h = q_all // ppr, q_all % ppr
+                    use = (row < rows_valid) & (8 * h < n)
+                    inside(((k_base + row[use]) * n + 8 * h[use]) * 2, 16, b_size, "split-K kernel: padded B pieces")
+                elif mode == "b4":
+                    ppr = nc // 8
+                    row, h = q_all // ppr, q_all % ppr
+                    use = (row < rows_valid) & (h == 0)
+                    inside((k_base + row[use]) * 8, 8, b_size, "split-K kernel: 8-byte B rows")
+                else:  # element copies
+                    valid = rows_valid * n
+                    e = np.arange(img_rows * n)
+                    inside((k_base * n + e[e < valid]) * 2, 2, b_size, "split-K kernel: B elements")
+        # --- result: rows of the workgroup's row blocks, columns below n
+        rows_out = np.arange(rb_first * 32, min((rb_first + R) * 32, m))
+        cols = np.arange(n)
+        if tokens:
+            inside((cols[None, :] * m + rows_out[:, None]) * d_size, d_size, m * n * d_size, "split-K kernel: y")
+        else:
+            inside((rows_out[:, None] * n + cols[None, :]) * d_size, d_size, m * n * d_size, "split-K kernel: D")
+
+
+# ---------------------------------------------------------------------------------------------------------------
+def tile_of_block(b, tiles_m, tiles_n, group_m):
+    total = tiles_m * tiles_n
+    per, rem = total // 8, total % 8
+    x, local = b % 8, b // 8
+    v = x * per + min(x, rem) + local
+    strip = v // (tiles_m * 4)
+    strip_w = min(tiles_n - strip * 4, 4)
+    w = v - strip * 4 * tiles_m
+    group = w // (group_m * strip_w)
+    group_h = min(tiles_m - group * group_m, group_m)
+    u = w - group * group_m * strip_w
+    return group * group_m + u % group_h, strip * 4 + u // group_h
+
+
+def check_gemm(m, n, k, tile, splits, pad_b, tokens=False, b_aligned=True, d_size=2):
+    WM, WN, FM, FN, KG = TILES[tile]
+    aligned = tokens or pad_b or (n % 8 == 0 and b_aligned)
+    if not aligned:
+        WM, WN, FM, FN, KG = 4, 1, 1, 4, 1  # the element-copy variant
+    BM, BN, NW = WM * FM * 32, WN * FN * 32, WM * WN * KG
+    CH = BN // 8
+    NL = STAGE_K * CH // (64 * NW)
+    NA = ((BM // 32) * BLOCK + 1024 * NW - 1) // (1024 * NW)
+    tiles_m, tiles_n = (m + BM - 1) // BM, (n + BN - 1) // BN
+    chunks_total = (k + 255) // 256
+    prep_size = prepared_bytes(m, k)
+    assert prep_size < (1 << 32)  # 32-bit copy offsets (the C ABI refuses larger weights)
+    cps = (chunks_total + splits - 1) // splits
+    splits = (chunks_total + cps - 1) // cps
+    assert (splits - 1) * cps < chunks_total  # the launcher's check: no empty split
+    ldb = k if tokens else ((n + 7) // 8 * 8 if pad_b else n)
+    b_size = (n * k if tokens else k * ldb) * 2
+    if tokens:
+        assert k * 256 * 2 < (1 << 32)
+    # the workgroup -> tile mapping is a bijection
+    seen = {tile_of_block(b, tiles_m, tiles_n, 8 if NW == 8 else 16) for b in range(tiles_m * tiles_n)}
+    assert seen == {(tm, tn) for tm in range(tiles_m) for tn in range(tiles_n)}
+    rb_total = m // 32
+    corner_tiles = {(0, 0), (tiles_m - 1, 0), (0, tiles_n - 1), (tiles_m - 1, tiles_n - 1), (tiles_m // 2, tiles_n // 2)}
+    for split in sorted({0, splits - 1, splits // 2}):
+        chunk_begin = split * cps
+        chunk_end = min(chunk_begin + cps, chunks_total)
+        for tile_m, tile_n in corner_tiles:
+            n0 = tile_n * BN
+            if aligned:
+                for wave in range(NW):
+                    for i in range(NL):
+                        slot = (NW * i + wave) * 64 + LANE
+                        if tokens:
+                            token = slot // 8
+                            sw = np.where(True, (token >> 1) & 7, 0)
+                            lc = (slot % 8) ^ sw
+                            token = np.where(n0 + token >= n, 0, token)
+                            b_off = (token * k + 8 * lc) * 2
+                            copy_row = 8 * lc
+                            stage_stride, stage0 = STAGE_K * 2, n0 * k * 2
+                        else:
+                            row, pc = slot // CH, slot % CH
+                            sw = ((row & 3) << 2) if BN >= 128 else (((row >> 1) & 1) << 2)
+                            lc = pc ^ sw
+                            col = np.where(n0 + 8 * lc >= ldb, 0, 8 * lc)
+                            b_off = (row * ldb + col) * 2
+                            copy_row = row
+                            stage_stride, stage0 = STAGE_K * ldb * 2, n0 * 2
+                        assert b_off.max() < (1 << 32)
+                        # stages copied: the first four of the split's range, then four more per chunk of the loop
+                        for stage in range(chunk_begin * STAGES, chunk_end * STAGES + STAGES):
+                            next_k0 = stage * STAGE_K
+                            base = stage0 + stage * stage_stride
+                            if next_k0 + STAGE_K <= k:
+                                inside(base + b_off, 16, b_size, "main kernel: B stage copy")
+                            else:
+                                real = next_k0 + copy_row < k  # the other lanes copy from the block of zeros
+                                inside(base + b_off[real], 16, b_size, "main kernel: B stage copy (K tail)")
+                    rb0 = tile_m * (BM // 32)
+                    for j in range(NA):
+                        byte = (NW * j + wave) * 1024 + LANE * 16
+                        blk, off = byte // BLOCK, byte % BLOCK
+                        blk = np.where(blk >= BM // 32, 0, blk)
+                        rb = np.minimum(rb0 + blk, rb_total - 1)
+                        a_off = rb * chunks_total * BLOCK + off
+                        # the chunk pointer advances while next_chunk + 1 < chunks: it never passes the last chunk
+                        for chunk in range(chunk_begin, min(chunk_end + 1, chunks_total)):
+                            inside(chunk * BLOCK + a_off, 16, prep_size, "main kernel: prepared block copy")
+            else:
+                rows_k = np.arange(k)
+                cols = n0 + np.arange(BN)
+                cols = cols[cols < n]
+                inside((rows_k[:, None] * n + cols[None, :]) * 2, 2, k * n * 2, "main kernel: B elements")
+                for fm in range(FM):
+                    for wm in range(WM):
+                        rb = min((tile_m * BM + wm * FM * 32) // 32 + fm, rb_total - 1)
+                        for chunk in range(chunk_begin, chunk_end):
+                            base = rb * chunks_total * BLOCK + chunk * BLOCK
+                            inside(base + LANE * 16, 16, prep_size, "main kernel: prepared block (direct)")
+                            inside(base + SIGN_OFF + LANE * 8, 8, prep_size, "main kernel: prepared signs (direct)")
+            # result range of the tile: rows below m, columns below n, in this split's slice when K is split
+            rows_out = np.arange(tile_m * BM, min((tile_m + 1) * BM, m))
+            cols_out = np.arange(n0, min(n0 + BN, n))
+            elem = 4 if splits > 1 else d_size
+            slice0 = split * m * n * elem if splits > 1 else 0
+            total = (splits if splits > 1 else 1) * m * n * elem
+            if tokens:
+                inside(slice0 + (cols_out[None, :] * m + rows_out[:, None]) * elem, elem, total, "main kernel: y")
+            else:
+                inside(slice0 + (rows_out[:, None] * n + cols_out[None, :]) * elem, elem, total, "main kernel: D")
+    if splits > 1:  # splitk_reduce_kernel: one thread per 4 (or 1) results
+        total = m * n
+        vec = 4 if total % 4 == 0 else 1
+        first = (np.arange((total // vec + 255) // 256 * 256, dtype=np.int64)) * vec
+        first = first[first < total]
+        for s in (0, splits - 1):
+            inside((s * total + first) * 4, 4 * vec, splits * total * 4, "reduce: partial sums")
+        inside(first * d_size, d_size * vec, total * d_size, "reduce: result")
+    if pad_b:  # pad_b_kernel: one thread per 16-byte piece of the padded copy
+        pieces_per_row = ldb // 8
+        piece = np.arange(k * pieces_per_row, dtype=np.int64)
+        row, col0 = piece // pieces_per_row, (piece % pieces_per_row) * 8
+        for j in (0, 7):
+            ok = col0 + j < n
+            inside((row[ok] * n + col0[ok] + j) * 2, 2, k * n * 2, "pad_b: source")
+        inside((row * ldb + col0) * 2, 16, k * ldb * 2, "pad_b: destination")
+
+
+def check_call(m, n, k, tokens=False, b_aligned=True):
+    plan = _native.describe_launch(m, n, k, b_aligned=b_aligned or tokens)
+    if plan["kernel"] == "skinny_kernel":
+        check_skinny(m, n, k, plan["rows"], tokens=tokens, b_aligned=b_aligned)
+    else:
+        check_gemm(m, n, k, plan["tile"], plan["splits"], plan["pad_b"] and not tokens, tokens=tokens, b_aligned=b_aligned)
+    return plan
+
+
+@pytest.fixture()
+def hooks():
+    def reset():
+        _native.set_tile_config(-1)
+        _native.set_skinny_enabled(True)
+        _native.set_skinny_rows(-1)
+        _native.set_split_k(-1)
+        _native.set_pad_b(True)
+    reset()
+    yield
+    reset()
+
+
+@pytest.mark.parametrize("m,k", [(64, 32), (512, 512), (8192, 8192), (11008, 4096), (4096, 11008), (8192, 28672), (25600, 25600)])
+def test_prepare_kernel_addresses(m, k):
+    check_prepare(m, k)
+
+
+@pytest.mark.parametrize("n", [40, 48, 64])
+@pytest.mark.parametrize("rows,skinny", [(32, True), (64, True), (-1, False)])
+def test_long_k_wide_skinny_shapes(hooks, n, rows, skinny):
+    """8192 x 28672 with 33 to 64 columns: the 64-column images of the split-K kernel with 32- and 64-row workgroups, and
+    the main kernel with the K split its plan chooses, plain and token-major."""
+    m, k = 8192, 28672
+    _native.set_skinny_rows(rows)
+    _native.set_skinny_enabled(skinny)
+    for tokens in (False, True):
+        plan = check_call(m, n, k, tokens=tokens)
+        assert (plan["kernel"] == "skinny_kernel") == skinny
+
+
+@pytest.mark.parametrize("m,n,k", [(512, 512, 512), (1024, 1024, 1024), (2048, 2048, 2048), (4096, 4096, 4096), (8192, 8192, 8192),
+                                   (11008, 1, 4096), (11008, 4, 4096), (11008, 16, 4096), (4096, 1, 11008),
+                                   (4096, 4, 11008), (4096, 16, 11008), (4096, 2048, 4096), (16384, 16384, 16384),
+                                   (25600, 25600, 25600)])
+def test_benchmark_configurations(hooks, m, n, k):
+    check_call(m, n, k)
+    if n >= 16:
+        check_call(m, n, k, tokens=True)
+
+
+@pytest.mark.parametrize("m,n,k,b_aligned", [(64, 1, 32, True), (192, 5, 800, True), (320, 8, 4128, True), (128, 13, 12320, True),
+                                             (320, 17, 4128, True), (1088, 31, 2208, True), (64, 33, 32, True),
+                                             (1088, 63, 2208, True), (2048, 32, 20480, True), (4096, 16, 16384, True),
+                                             (576, 200, 352, True), (640, 1001, 160, True), (4096, 1001, 4096, True),
+                                             (256, 264, 512, False), (1024, 203, 4128, True), (128, 1000, 4128, True),
+                                             (28672, 40, 512, True), (20480, 64, 1024, True), (4096, 384, 11008, True),
+                                             (64, 72, 64, False), (2112, 1032, 64, True)])
+def test_ragged_and_split_shapes(hooks, m, n, k, b_aligned):
+    for rows in (-1, 32, 64, 128):
+        _native.set_skinny_rows(rows)
+        check_call(m, n, k, b_aligned=b_aligned)
+    _native.set_skinny_rows(-1)
+    check_call(m, n, k, tokens=True)
+    _native.set_skinny_enabled(False)
+    for splits in (-1, 1, 3, 16):
+        _native.set_split_k(splits)
+        check_call(m, n, k, b_aligned=b_aligned)
+        check_call(m, n, k, tokens=True)
+
+
+@pytest.mark.parametrize("tile", sorted(TILES))
+def test_every_tile_configuration(hooks, tile):
+    _native.set_tile_config(tile)
+    _native.set_skinny_enabled(False)
+    for m, n, k in ((1024, 512, 1024), (576, 264, 192), (2112, 1032, 64), (8192, 8192, 8192)):
+        check_call(m, n, k)
+        if tile in (4, 6, 9, 10, 11, 12, 13, 14):
+            check_call(m, n, k, tokens=True)
+
+
+def test_the_model_catches_an_out_of_range_access():
+    """the checker itself: a prepared operand one block too small, or B one row too short, must be flagged"""
+    with pytest.raises(AssertionError):
+        inside(np.array([0, prepared_bytes(64, 256) - 8]), 16, prepared_bytes(64, 256), "probe")
+    real = prepared_bytes
+
+    def short(m, k):
+        return real(m, k) - BLOCK
+    globals()["prepared_bytes"] = short
+    try:
+        with pytest.raises(AssertionError):
+            check_skinny(1024, 16, 4096, 64)
+        with pytest.raises(AssertionError):
+            check_gemm(1024, 512, 1024, 9, 1, False)
+    finally:
+        globals()["prepared_bytes"] = real
