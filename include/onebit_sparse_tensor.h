@@ -125,8 +125,9 @@ void onebit_sparse_set_tile_config(int tile_config);
 void onebit_sparse_set_skinny_enabled(int enabled);
 /* Weight rows one workgroup of the split-K kernel covers: 32, 64 or 128; <= 0 = automatic. */
 void onebit_sparse_set_skinny_rows(int rows);
-/* K splits of the main kernel (n > 16): 1 = never split, N > 1 = N splits (at most one per 256 of K), <= 0 =
- * automatic (few tiles and a long K). A split call writes fp32 partial sums to a library-owned buffer kept per
+/* K splits over workgroups, of the main kernel and of the split-K kernel (which also splits K among the wavefronts
+ * of a workgroup): 1 = never split, N > 1 = N splits (at most one per 256 of K), <= 0 = automatic (few tiles or row
+ * groups and a long K). A split call writes fp32 partial sums to a library-owned buffer kept per
  * device and stream (grown with hipMalloc on first use: warm up before capturing the call in a HIP graph) and adds
  * them in split order, so results do not depend on timing. */
 void onebit_sparse_set_split_k(int splits);
@@ -157,7 +158,7 @@ int onebit_sparse_release_buffers(void);
 /* Diagnostic, no counterpart in the reference, host-only (touches no GPU): what a prepared call of this shape would
  * launch under the calling thread's hooks on a GPU with 256 compute units (calls plan for the device they run on). plan[0] = 1 for the split-K kernel (n <= 64), 0 for the main kernel; plan[1] =
  * weight rows per workgroup (split-K kernel) or the tile code (main kernel); plan[2] = K splits over workgroups
- * (main kernel, 1 = none); plan[3] = 1 if B is read through a padded copy. */
+ * (1 = none); plan[3] = 1 if B is read through a padded copy. */
 int onebit_sparse_describe_launch(int m, int n, int k, int b_16_byte_aligned, int *plan);
 
 /* Diagnostic, no counterpart in the reference: sustained rate of v_smfmac_f32_32x32x32_f16 in a register-only

@@ -277,7 +277,7 @@ def describe_launch(m, n, k, b_aligned=True):
     plan = (ctypes.c_int * 4)()
     _check(lib().onebit_sparse_describe_launch(m, n, k, 1 if b_aligned else 0, plan))
     if plan[0]:
-        return dict(kernel="skinny_kernel", rows=plan[1])
+        return dict(kernel="skinny_kernel", rows=plan[1], splits=plan[2])
     return dict(kernel="gemm_kernel", tile=plan[1], splits=plan[2], pad_b=bool(plan[3]))
 
 

@@ -239,6 +239,45 @@ struct LaunchPlan {
   int pad_b;           // gemm_kernel: B is read through a padded copy
 };
 
+// Row group and K splits over workgroups of the split-K kernel. Every workgroup of that kernel reads all of B's rows
+// of its K range, so with few row groups over a long K (4096 x 28672 x 16: 128 workgroups that each read 900 KB of B
+// for 170 KB of weights) the compute units spend their time re-reading B and half of them have no workgroup at all.
+// Splitting K over S workgroups per row group divides both; the price is a second launch that adds the S partial
+// results (about 3 us in all). Rule fitted to a sweep of m = 2048 ... 11008, k = 4096 ... 28672, n = 16, 32, 64 over
+// every row group and S = 1 ... 8 (us, unsplit -> split): 2048 x 28672 x 16 18.5 -> 9.2, 4096 x 16384 x 16 12.0 -> 9.1,
+// 4096 x 28672 x 32 28.0 -> 15.6, 8192 x 28672 x 16 21.4 -> 18.4, 8192 x 16384 x 64 30.2 -> 23.0, 11008 x 28672 x 32
+// 34.2 -> 28.9; the best split always has at most one workgroup per compute unit and 64-row groups (128 rows when 64
+// rows leave no room for two splits); below the threshold on B's bytes per workgroup the second launch costs more
+// than the split saves (4096 x 11008 x 16: 8.9 against 8.5).
+struct SkinnyPlan {
+  int rows, splits;
+};
+SkinnyPlan plan_skinny(int m, int n, int k, int compute_units) {
+  const int chunks = (k + onebit::kChunkK - 1) / onebit::kChunkK;
+  const int forced_rows = g_skinny_rows, forced_splits = g_split_k;
+  // the largest row group that still gives about two workgroups per three compute units (measured: larger groups
+  // re-read B less often, but idle compute units cost more)
+  // (n > 32: two column fragments per row block, at most two row blocks per wavefront)
+  const int enough = std::max(1, 160 * compute_units / 256);
+  int rows = forced_rows > 0 ? forced_rows : (m / 128 >= enough && n <= 32) ? 128 : (m / 64 >= enough) ? 64 : 32;
+  if (forced_splits >= 1) return SkinnyPlan{rows, forced_splits > chunks ? chunks : forced_splits};
+  const double image_row_bytes = n <= 16 ? 32.0 : n <= 32 ? 64.0 : 128.0;
+  const double threshold = 400e3 * std::max(1.0, m / 4096.0);
+  if (chunks < 32 || k * image_row_bytes < threshold) return SkinnyPlan{rows, 1};
+  auto splits_for = [&](int r) {
+    const int groups = (m + r - 1) / r;
+    return std::min(compute_units / groups, chunks / 8);  // one workgroup per compute unit, eight chunks per workgroup
+  };
+  if (forced_rows > 0) {
+    const int s = splits_for(rows);
+    return SkinnyPlan{rows, s >= 2 ? s : 1};
+  }
+  if (const int s = splits_for(64); s >= 2) return SkinnyPlan{64, s};
+  if (n <= 32)
+    if (const int s = splits_for(128); s >= 2) return SkinnyPlan{128, s};
+  return SkinnyPlan{rows, 1};
+}
+
 LaunchPlan choose_launch(int m, int n, int k, bool b_16_byte_aligned, int compute_units = 256) {
   LaunchPlan plan{};
   // 32 < n <= 64: every 64-row workgroup of the split-K kernel stages all of B, which the main kernel's tiles overtake
@@ -246,15 +285,10 @@ LaunchPlan choose_launch(int m, int n, int k, bool b_16_byte_aligned, int comput
   // against 34.4; 65536 x 8192 66 against 68, at n = 40 77 against 66; 131072 x 2048 51 against 35)
   const bool skinny_shape = n <= 32 || (n <= onebit::kSkinnyMaxN && m <= 40960);
   if (skinny_shape && g_skinny_enabled) {
-    int rows = g_skinny_rows;
-    // the largest row group that still gives about two workgroups per three compute units (measured: larger groups
-    // re-read B less often, but idle compute units cost more)
-    // (n > 32: two column fragments per row block, at most two row blocks per wavefront)
-    const int enough = std::max(1, 160 * compute_units / 256);  // about two workgroups per three compute units
-    if (rows <= 0) rows = (m / 128 >= enough && n <= 32) ? 128 : (m / 64 >= enough) ? 64 : 32;
+    const SkinnyPlan sk = plan_skinny(m, n, k, compute_units);
     plan.split_k_kernel = 1;
-    plan.rows_or_tile = rows;
-    plan.splits = 1;
+    plan.rows_or_tile = sk.rows;
+    plan.splits = sk.splits;
     return plan;
   }
   const GemmPlan gemm = plan_gemm(m, n, k, compute_units);
@@ -274,6 +308,35 @@ struct FixedScratch {
   size_t bytes;
 };
 
+// K split of a split-K kernel launch: the split geometry and the partial-sum buffer (the caller's fixed workspace, or
+// the library-owned buffer of this device and stream).
+int setup_skinny_split(onebit::SkinnyArgs& args, int splits, hipStream_t stream, const FixedScratch* fixed) {
+  args.splits = 1;
+  if (splits <= 1) return ONEBIT_OK;
+  const int cps = (args.kc_total + splits - 1) / splits;
+  args.chunks_per_split = cps;
+  args.splits = (args.kc_total + cps - 1) / cps;  // every split non-empty
+  if (args.splits <= 1) return ONEBIT_OK;
+  const size_t bytes = (size_t)args.splits * args.m * args.n * sizeof(float);
+  if (fixed) {
+    if (bytes > fixed->bytes)
+      return fail(ONEBIT_ERR_ARGUMENT,
+                  "this shape needs %zu bytes of scratch (%d K splits of %d x %d fp32 partial sums); the static "
+                  "workspace of the non-allocating entry point holds %zu", bytes, args.splits, args.m, args.n, fixed->bytes);
+    args.split_ws = reinterpret_cast<float*>(fixed->base);
+    return ONEBIT_OK;
+  }
+  int device = 0;
+  ONEBIT_HIP(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) return fail(ONEBIT_ERR_ARGUMENT, "device ordinal %d not supported", device);
+  DeviceState& st = g_dev[device];
+  std::lock_guard<std::recursive_mutex> lock(st.mu);
+  Buffer& ws = st.split_ws[stream];
+  if (int rc = grow(&ws.ptr, &ws.bytes, bytes, stream); rc != ONEBIT_OK) return rc;
+  args.split_ws = static_cast<float*>(ws.ptr);
+  return ONEBIT_OK;
+}
+
 int matmul_prepared_impl(const void* prepared, const void* b, const void* c, void* d, int m, int n, int k, float alpha,
                          float beta, int c_dtype, int d_dtype, hipStream_t stream, const FixedScratch* fixed = nullptr) {
   if (!prepared || !b || !d) return fail(ONEBIT_ERR_ARGUMENT, "null operand pointer");
@@ -292,6 +355,7 @@ int matmul_prepared_impl(const void* prepared, const void* b, const void* c, voi
     args.alpha = alpha; args.beta = beta;
     args.c_f16 = c_dtype == ONEBIT_DTYPE_F16;
     args.d_f16 = d_dtype == ONEBIT_DTYPE_F16;
+    if (int rc = setup_skinny_split(args, plan.splits, stream, fixed); rc != ONEBIT_OK) return rc;
     ONEBIT_HIP(onebit::launch_skinny(args, plan.rows_or_tile, stream));
     return ONEBIT_OK;
   }
@@ -467,6 +531,7 @@ int onebit_sparse_linear_prepared(const void* prepared, const void* x, const voi
     args.d_f16 = y_dtype == ONEBIT_DTYPE_F16;
     args.bias = bias;
     args.bias_f16 = bias_dtype == ONEBIT_DTYPE_F16;
+    if (int rc = setup_skinny_split(args, plan.splits, static_cast<hipStream_t>(stream), nullptr); rc != ONEBIT_OK) return rc;
     ONEBIT_HIP(onebit::launch_skinny_tokens(args, plan.rows_or_tile, static_cast<hipStream_t>(stream)));
     return ONEBIT_OK;
   }

@@ -1215,25 +1215,31 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   // Short K (at most two chunks per wavefront, e.g. 11008 x 4096): everything the wavefront will read is requested
   // at once, so the kernel pays one memory latency instead of one per chunk.
   constexpr bool kShortPath = NW <= 8 && SUB == 1 && MODE != kSkinnyBScalar;
-  const bool short_k = kShortPath && kc_total <= 2 * NW;
+  // K split over workgroups (grid.y > 1): this workgroup multiplies the chunks [kc_begin, kc_end) and writes raw fp32
+  // sums to its slice of the partial-sum buffer; a second kernel adds the slices in order and applies the epilogue.
+  const int kc_begin = blockIdx.y * p.chunks_per_split;
+  const int kc_end = kc_begin + p.chunks_per_split < kc_total ? kc_begin + p.chunks_per_split : kc_total;
+  char* const d_out = reinterpret_cast<char*>(p.d) + (size_t)blockIdx.y * p.m * p.n * (p.d_f16 ? 2 : 4);
+  const int first = kc_begin + wave;  // this wavefront's first chunk
+  const bool short_k = kShortPath && kc_end - kc_begin <= 2 * NW;
   if (short_k) {
     u32x4_t breg2[8];
-    load_b(wave * kChunkK, breg);
-    load_a(wave, a_cur);
-    load_b((wave + NW) * kChunkK, breg2);  // all zeros when the wavefront has one chunk only
-    load_a(wave + NW, a_next);
-    if (wave < kc_total) {
-      store_b(wave * kChunkK, breg);
+    load_b(first * kChunkK, breg);
+    load_a(first, a_cur);
+    load_b((first + NW) * kChunkK, breg2);
+    load_a(first + NW, a_next);
+    if (first < kc_end) {
+      store_b(first * kChunkK, breg);
       compute(a_cur, std::integral_constant<int, 0>{});
     }
-    if (wave + NW < kc_total) {
-      store_b((wave + NW) * kChunkK, breg2);
+    if (first + NW < kc_end) {
+      store_b((first + NW) * kChunkK, breg2);
       compute(a_next, std::integral_constant<int, 0>{});
     }
   }
-  if (kPrefetchB && !short_k) load_b(wave * kChunkK, breg);
-  if (!short_k) load_a(wave, a_cur);
-  for (int kc = short_k ? kc_total : wave; kc < kc_total; kc += NW) {
+  if (kPrefetchB && !short_k) load_b(first * kChunkK, breg);
+  if (!short_k) load_a(first, a_cur);
+  for (int kc = short_k ? kc_end : first; kc < kc_end; kc += NW) {
     const int k_base = kc * kChunkK;
     if (!kPrefetchB) load_b(k_base, breg);
     store_b(k_base, breg);  // after the previous image's fragment reads: LDS operations of a wavefront execute in order
@@ -1300,8 +1306,8 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
           if (p.bias) sum += p.bias_f16 ? (float)reinterpret_cast<const _Float16*>(p.bias)[row]
                                         : reinterpret_cast<const float*>(p.bias)[row];
           const size_t o = (size_t)token * p.m + row;
-          if (p.d_f16) reinterpret_cast<_Float16*>(p.d)[o] = (_Float16)sum;
-          else reinterpret_cast<float*>(p.d)[o] = sum;
+          if (p.d_f16) reinterpret_cast<_Float16*>(d_out)[o] = (_Float16)sum;
+          else reinterpret_cast<float*>(d_out)[o] = sum;
         }
       }
     } else {
@@ -1318,8 +1324,8 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
             const float cv = p.c_f16 ? (float)reinterpret_cast<const _Float16*>(p.c)[o] : reinterpret_cast<const float*>(p.c)[o];
             x = x + p.beta * cv;
           }
-          if (p.d_f16) reinterpret_cast<_Float16*>(p.d)[o] = (_Float16)x;
-          else reinterpret_cast<float*>(p.d)[o] = x;
+          if (p.d_f16) reinterpret_cast<_Float16*>(d_out)[o] = (_Float16)x;
+          else reinterpret_cast<float*>(d_out)[o] = x;
         }
       }
     }
@@ -1395,6 +1401,22 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     if (d_f16) reinterpret_cast<_Float16*>(d)[first] = (_Float16)x[0];
     else reinterpret_cast<float*>(d)[first] = x[0];
   }
+}
+
+// Second pass of a K split: ordered sum of the partial results and the epilogue (bias and row_length for the
+// token-major form, where element i of y takes bias[i % m]).
+static hipError_t launch_split_reduce(const float* ws, int splits, size_t total, const void* c, void* d, float alpha,
+                                      float beta, int c_f16, int d_f16, const void* bias, int bias_f16, int row_length,
+                                      hipStream_t stream) {
+  const bool vec = total % 4 == 0 && (reinterpret_cast<uintptr_t>(d) & 15) == 0 &&
+                   (beta == 0.f || (reinterpret_cast<uintptr_t>(c) & 15) == 0) && (!bias || row_length % 4 == 0);
+  if (vec)
+    hipLaunchKernelGGL(splitk_reduce_kernel<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream, ws,
+                       splits, total, c, d, total, alpha, beta, c_f16, d_f16, bias, bias_f16, row_length);
+  else
+    hipLaunchKernelGGL(splitk_reduce_kernel<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, ws,
+                       splits, total, c, d, total, alpha, beta, c_f16, d_f16, bias, bias_f16, row_length);
+  return hipGetLastError();
 }
 
 // =====================================================================================================
@@ -1500,17 +1522,8 @@ hipError_t launch_gemm_tokens(GemmArgs args, int tile_config, hipStream_t stream
   first.d_f16 = 0;
   first.bias = nullptr;
   if (hipError_t st = pass(first); st != hipSuccess) return st;
-  const size_t total = (size_t)args.m * args.n;
-  const bool vec = (reinterpret_cast<uintptr_t>(args.d) & 15) == 0;  // m is a multiple of 64
-  if (vec)
-    hipLaunchKernelGGL(splitk_reduce_kernel<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream,
-                       args.split_ws, args.splits, total, nullptr, args.d, total, 1.f, 0.f, 0, args.d_f16, args.bias,
-                       args.bias_f16, args.m);
-  else
-    hipLaunchKernelGGL(splitk_reduce_kernel<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
-                       args.split_ws, args.splits, total, nullptr, args.d, total, 1.f, 0.f, 0, args.d_f16, args.bias,
-                       args.bias_f16, args.m);
-  return hipGetLastError();
+  return launch_split_reduce(args.split_ws, args.splits, (size_t)args.m * args.n, nullptr, args.d, 1.f, 0.f, 0, args.d_f16,
+                             args.bias, args.bias_f16, args.m, stream);
 }
 
 hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
@@ -1542,24 +1555,15 @@ hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream) {
   pass.d = args.split_ws;
   pass.d_f16 = 0;
   if (hipError_t st = launch_gemm_pass(pass, tile_config, stream); st != hipSuccess) return st;
-  const size_t total = (size_t)args.m * args.n;
-  const bool vec = total % 4 == 0 && (reinterpret_cast<uintptr_t>(args.d) & 15) == 0 &&
-                   (args.beta == 0.f || (reinterpret_cast<uintptr_t>(args.c) & 15) == 0);
-  if (vec)
-    hipLaunchKernelGGL(splitk_reduce_kernel<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream,
-                       args.split_ws, args.splits, total, args.c, args.d, total, args.alpha, args.beta, args.c_f16,
-                       args.d_f16, nullptr, 0, 1);
-  else
-    hipLaunchKernelGGL(splitk_reduce_kernel<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
-                       args.split_ws, args.splits, total, args.c, args.d, total, args.alpha, args.beta, args.c_f16,
-                       args.d_f16, nullptr, 0, 1);
-  return hipGetLastError();
+  return launch_split_reduce(args.split_ws, args.splits, (size_t)args.m * args.n, args.c, args.d, args.alpha, args.beta,
+                             args.c_f16, args.d_f16, nullptr, 0, 1, stream);
 }
 
 template <int NW, int R, int MODE, int NC>
 static hipError_t launch_skinny_mode(const SkinnyArgs& args, hipStream_t stream) {
   const int row_blocks = args.m / kRowBlock;
-  hipLaunchKernelGGL((skinny_kernel<NW, R, MODE, NC>), dim3((row_blocks + R - 1) / R), dim3(64 * NW), 0, stream, args);
+  hipLaunchKernelGGL((skinny_kernel<NW, R, MODE, NC>), dim3((row_blocks + R - 1) / R, args.splits), dim3(64 * NW), 0,
+                     stream, args);
   return hipGetLastError();
 }
 
@@ -1591,26 +1595,58 @@ static hipError_t launch_skinny_tokens_cfg(const SkinnyArgs& args, hipStream_t s
   return launch_skinny_mode<NW, R, kSkinnyBTokens, 16>(args, stream);
 }
 
+// Fills in the K split of a split-K kernel launch: splits <= 1 = one pass straight into d.
+static hipError_t skinny_split_setup(SkinnyArgs& args, SkinnyArgs& first_pass) {
+  if (args.splits <= 1) {
+    args.splits = 1;
+    args.chunks_per_split = args.kc_total;
+    first_pass = args;
+    return hipSuccess;
+  }
+  if (args.chunks_per_split < 1 || (long)(args.splits - 1) * args.chunks_per_split >= args.kc_total || !args.split_ws)
+    return hipErrorInvalidValue;  // an empty split would only add zeros, but it is a planning error
+  first_pass = args;  // raw fp32 partial sums per split, laid out like the result
+  first_pass.alpha = 1.f;
+  first_pass.beta = 0.f;
+  first_pass.c = nullptr;
+  first_pass.bias = nullptr;
+  first_pass.d = args.split_ws;
+  first_pass.d_f16 = 0;
+  return hipSuccess;
+}
+
 hipError_t launch_skinny_tokens(SkinnyArgs args, int rows_per_group, hipStream_t stream) {
   if (args.n < 1 || args.n > kSkinnyMaxN) return hipErrorInvalidValue;
   // 16-byte loads of x; lane offsets of up to 64 token rows must stay below the "outside" offset of the kernel
   if ((reinterpret_cast<uintptr_t>(args.b) & 15) != 0 || (size_t)args.k * 64 * 2 >= 0xFFFFFF00u) return hipErrorInvalidValue;
+  SkinnyArgs pass;
+  if (hipError_t st = skinny_split_setup(args, pass); st != hipSuccess) return st;
+  hipError_t st;
   switch (rows_per_group) {
-    case 32: return launch_skinny_tokens_cfg<16, 1>(args, stream);
-    case 64: return launch_skinny_tokens_cfg<8, 2>(args, stream);
-    case 128: return launch_skinny_tokens_cfg<8, 4>(args, stream);
+    case 32: st = launch_skinny_tokens_cfg<16, 1>(pass, stream); break;
+    case 64: st = launch_skinny_tokens_cfg<8, 2>(pass, stream); break;
+    case 128: st = launch_skinny_tokens_cfg<8, 4>(pass, stream); break;
     default: return hipErrorInvalidValue;
   }
+  if (st != hipSuccess || args.splits <= 1) return st;
+  return launch_split_reduce(args.split_ws, args.splits, (size_t)args.m * args.n, nullptr, args.d, 1.f, 0.f, 0, args.d_f16,
+                             args.bias, args.bias_f16, args.m, stream);
 }
 
 hipError_t launch_skinny(SkinnyArgs args, int rows_per_group, hipStream_t stream) {
   if (args.n < 1 || args.n > kSkinnyMaxN) return hipErrorInvalidValue;
+  SkinnyArgs pass;
+  if (hipError_t st = skinny_split_setup(args, pass); st != hipSuccess) return st;
+  hipError_t st;
   switch (rows_per_group) {
-    case 32: return launch_skinny_cfg<16, 1>(args, stream);  // sixteen wavefronts split K: small M
-    case 64: return launch_skinny_cfg<8, 2>(args, stream);
-    case 128: return launch_skinny_cfg<8, 4>(args, stream);  // n > 32: 64-row groups
+    case 32: st = launch_skinny_cfg<16, 1>(pass, stream); break;  // sixteen wavefronts split K: small M
+    case 64: st = launch_skinny_cfg<8, 2>(pass, stream); break;
+    case 128: st = launch_skinny_cfg<8, 4>(pass, stream); break;  // n > 32: 64-row groups
     default: return hipErrorInvalidValue;
   }
+  if (st != hipSuccess || args.splits <= 1) return st;
+  return launch_split_reduce(args.split_ws, args.splits, (size_t)args.m * args.n, args.c, args.d, args.alpha, args.beta,
+                             args.c_f16, args.d_f16, nullptr, 0, 1, stream);
 }
 
 }  // namespace onebit

@@ -46,6 +46,12 @@ struct SkinnyArgs {
   // not used, bias (m values, may be null) is added to every token's row
   const void* bias;
   int bias_f16;
+  // K split over workgroups (grid.y = splits), for few row groups over a long K: split s multiplies the K chunks
+  // [s * chunks_per_split, +chunks_per_split) and writes raw fp32 sums to split_ws + s * m * n (laid out like the
+  // result); a second kernel adds the splits in order and applies the epilogue. splits <= 1: one pass straight into d.
+  int splits;
+  int chunks_per_split;
+  float* split_ws;
 };
 
 enum TileConfig { kTile512x128 = 0, kTile256x128 = 1, kTile128x128 = 2, kTile256x256 = 3, kTile256x128w = 4, kTile512x128t = 5, kTile128x128s = 6, kTile256x64 = 7, kTile256x256w8 = 8, kTile512x128w8 = 9, kTile256x128w8 = 10, kTile128x128w8 = 11, kTile64x128 = 12, kTile128x128k2 = 13, kTile64x128k2 = 14, kTileAuto = -1 };

@@ -82,7 +82,7 @@ def skinny_variant(n, rows, b_aligned=True, tokens=False):
     return nw, r, nc, mode
 
 
-def check_skinny(m, n, k, rows, tokens=False, b_aligned=True, d_size=2):
+def check_skinny(m, n, k, rows, tokens=False, b_aligned=True, d_size=2, splits=1):
     nw, R, nc, mode = skinny_variant(n, rows, b_aligned, tokens)
     kc_total, rb_total = (k + 255) // 256, m // 32
     img_rows = 8192 // (nc * 2)
@@ -90,21 +90,28 @@ def check_skinny(m, n, k, rows, tokens=False, b_aligned=True, d_size=2):
     prep_size, b_size = prepared_bytes(m, k), k * n * 2
     grid = (rb_total + R - 1) // R
     prefetch_b = nw <= 8 and mode != "scalar"
-    short_k = nw <= 8 and sub == 1 and mode != "scalar" and kc_total <= 2 * nw
+    cps = (kc_total + splits - 1) // splits if splits > 1 else kc_total
+    splits = (kc_total + cps - 1) // cps
+    assert (splits - 1) * cps < kc_total  # the launcher's check: no empty split
     b_fits = b_size < (1 << 32)
     if tokens:
         assert k * 64 * 2 < 0xFFFFFF00  # the launcher's check
-    for wg in sorted({0, 1, grid // 2, grid - 1} & set(range(grid))):
+    for wg, split in [(g, sp) for g in sorted({0, 1, grid // 2, grid - 1} & set(range(grid)))
+                      for sp in sorted({0, splits // 2, splits - 1})]:
         rb_first = wg * R
+        kc_begin = split * cps
+        kc_end = min(kc_begin + cps, kc_total)
+        short_k = nw <= 8 and sub == 1 and mode != "scalar" and kc_end - kc_begin <= 2 * nw
         for wave in range(nw):
+            first = kc_begin + wave
             # --- prepared operand through one descriptor per row block
             chunks = []
             if short_k:
-                chunks += [wave, wave + nw]
+                chunks += [first, first + nw]
             else:
-                chunks.append(wave)
-                kc = wave
-                while kc < kc_total:
+                chunks.append(first)
+                kc = first
+                while kc < kc_end:
                     chunks.append(kc + nw)
                     kc += nw
             for r in range(R):
@@ -119,12 +126,12 @@ def check_skinny(m, n, k, rows, tokens=False, b_aligned=True, d_size=2):
             # --- B images
             k_bases = []
             if short_k:
-                k_bases += [wave * CHUNK_K, (wave + nw) * CHUNK_K]
+                k_bases += [first * CHUNK_K, (first + nw) * CHUNK_K]
             else:
-                kc = wave
+                kc = first
                 if prefetch_b:
-                    k_bases.append(wave * CHUNK_K)
-                while kc < kc_total:
+                    k_bases.append(first * CHUNK_K)
+                while kc < kc_end:
                     for s in range(sub):
                         k_bases.append(kc * CHUNK_K + s * img_rows)
                     if prefetch_b:
@@ -178,10 +185,26 @@ def check_skinny(m, n, k, rows, tokens=False, b_aligned=True, d_size=2):
         # --- result: rows of the workgroup's row blocks, columns below n
         rows_out = np.arange(rb_first * 32, min((rb_first + R) * 32, m))
         cols = np.arange(n)
+        elem = 4 if splits > 1 else d_size          # a split writes fp32 partial sums to its slice of the workspace
+        slice0 = split * m * n * elem if splits > 1 else 0
+        total = splits * m * n * elem
         if tokens:
-            inside((cols[None, :] * m + rows_out[:, None]) * d_size, d_size, m * n * d_size, "split-K kernel: y")
+            inside(slice0 + (cols[None, :] * m + rows_out[:, None]) * elem, elem, total, "split-K kernel: y")
         else:
-            inside((rows_out[:, None] * n + cols[None, :]) * d_size, d_size, m * n * d_size, "split-K kernel: D")
+            inside(slice0 + (rows_out[:, None] * n + cols[None, :]) * elem, elem, total, "split-K kernel: D")
+    if splits > 1:
+        check_reduce(m, n, splits, d_size)
+
+
+def check_reduce(m, n, splits, d_size):
+    """splitk_reduce_kernel: one thread per 4 (or 1) results"""
+    total = m * n
+    vec = 4 if total % 4 == 0 else 1
+    first = (np.arange((total // vec + 255) // 256 * 256, dtype=np.int64)) * vec
+    first = first[first < total]
+    for s in (0, splits - 1):
+        inside((s * total + first) * 4, 4 * vec, splits * total * 4, "reduce: partial sums")
+    inside(first * d_size, d_size * vec, total * d_size, "reduce: result")
 
 
 # ---------------------------------------------------------------------------------------------------------------
@@ -291,14 +314,8 @@ def check_gemm(m, n, k, tile, splits, pad_b, tokens=False, b_aligned=True, d_siz
                 inside(slice0 + (cols_out[None, :] * m + rows_out[:, None]) * elem, elem, total, "main kernel: y")
             else:
                 inside(slice0 + (rows_out[:, None] * n + cols_out[None, :]) * elem, elem, total, "main kernel: D")
-    if splits > 1:  # splitk_reduce_kernel: one thread per 4 (or 1) results
-        total = m * n
-        vec = 4 if total % 4 == 0 else 1
-        first = (np.arange((total // vec + 255) // 256 * 256, dtype=np.int64)) * vec
-        first = first[first < total]
-        for s in (0, splits - 1):
-            inside((s * total + first) * 4, 4 * vec, splits * total * 4, "reduce: partial sums")
-        inside(first * d_size, d_size * vec, total * d_size, "reduce: result")
+    if splits > 1:
+        check_reduce(m, n, splits, d_size)
     if pad_b:  # pad_b_kernel: one thread per 16-byte piece of the padded copy
         pieces_per_row = ldb // 8
         piece = np.arange(k * pieces_per_row, dtype=np.int64)
@@ -312,7 +329,7 @@ def check_gemm(m, n, k, tile, splits, pad_b, tokens=False, b_aligned=True, d_siz
 def check_call(m, n, k, tokens=False, b_aligned=True):
     plan = _native.describe_launch(m, n, k, b_aligned=b_aligned or tokens)
     if plan["kernel"] == "skinny_kernel":
-        check_skinny(m, n, k, plan["rows"], tokens=tokens, b_aligned=b_aligned)
+        check_skinny(m, n, k, plan["rows"], tokens=tokens, b_aligned=b_aligned, splits=plan["splits"])
     else:
         check_gemm(m, n, k, plan["tile"], plan["splits"], plan["pad_b"] and not tokens, tokens=tokens, b_aligned=b_aligned)
     return plan
@@ -365,13 +382,21 @@ def test_benchmark_configurations(hooks, m, n, k):
                                              (576, 200, 352, True), (640, 1001, 160, True), (4096, 1001, 4096, True),
                                              (256, 264, 512, False), (1024, 203, 4128, True), (128, 1000, 4128, True),
                                              (28672, 40, 512, True), (20480, 64, 1024, True), (4096, 384, 11008, True),
-                                             (64, 72, 64, False), (2112, 1032, 64, True)])
+                                             (64, 72, 64, False), (2112, 1032, 64, True), (4096, 16, 16384, True),
+                                             (2048, 33, 28672, True), (11008, 32, 28672, True), (192, 5, 12320, True)])
 def test_ragged_and_split_shapes(hooks, m, n, k, b_aligned):
     for rows in (-1, 32, 64, 128):
         _native.set_skinny_rows(rows)
         check_call(m, n, k, b_aligned=b_aligned)
     _native.set_skinny_rows(-1)
     check_call(m, n, k, tokens=True)
+    for splits in (2, 3, 16):  # the split-K kernel's own K split over workgroups (n <= 64), forced
+        _native.set_split_k(splits)
+        for rows in (32, 64, 128):
+            _native.set_skinny_rows(rows)
+            check_call(m, n, k, b_aligned=b_aligned)
+            check_call(m, n, k, tokens=True)
+    _native.set_skinny_rows(-1)
     _native.set_skinny_enabled(False)
     for splits in (-1, 1, 3, 16):
         _native.set_split_k(splits)

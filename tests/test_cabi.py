@@ -136,14 +136,22 @@ def test_launch_plan_of_the_benchmark_shapes(_default_hooks):
     assert plan(512, 512, 512) == dict(kernel="gemm_kernel", tile=12, splits=1, pad_b=False)
     # decode shapes: the split-K kernel, row group by M
     for n in (1, 4, 16):
-        assert plan(11008, n, 4096) == dict(kernel="skinny_kernel", rows=64)
-        assert plan(4096, n, 11008) == dict(kernel="skinny_kernel", rows=32)
-    assert plan(28672, 16, 8192) == dict(kernel="skinny_kernel", rows=128)
-    assert plan(28672, 32, 8192) == dict(kernel="skinny_kernel", rows=128)
-    assert plan(16384, 32, 4096) == dict(kernel="skinny_kernel", rows=64)
-    assert plan(4096, 64, 4096) == dict(kernel="skinny_kernel", rows=32)
-    assert plan(11008, 64, 4096) == dict(kernel="skinny_kernel", rows=64)   # 33 ... 64 columns: at most 64 rows
-    assert plan(28672, 64, 8192) == dict(kernel="skinny_kernel", rows=64)
+        assert plan(11008, n, 4096) == dict(kernel="skinny_kernel", rows=64, splits=1)
+        assert plan(4096, n, 11008) == dict(kernel="skinny_kernel", rows=32, splits=1)
+    assert plan(28672, 16, 8192) == dict(kernel="skinny_kernel", rows=128, splits=1)
+    assert plan(28672, 32, 8192) == dict(kernel="skinny_kernel", rows=128, splits=1)
+    assert plan(16384, 32, 4096) == dict(kernel="skinny_kernel", rows=64, splits=1)
+    assert plan(4096, 64, 4096) == dict(kernel="skinny_kernel", rows=32, splits=1)
+    assert plan(11008, 64, 4096) == dict(kernel="skinny_kernel", rows=64, splits=1)   # 33 ... 64 columns: at most 64 rows
+    assert plan(28672, 64, 8192) == dict(kernel="skinny_kernel", rows=64, splits=1)
+    # few row groups over a long K: K split over workgroups as well, one workgroup per compute unit, 64-row groups
+    assert plan(4096, 16, 16384) == dict(kernel="skinny_kernel", rows=64, splits=4)
+    assert plan(2048, 16, 28672) == dict(kernel="skinny_kernel", rows=64, splits=8)
+    assert plan(8192, 16, 28672) == dict(kernel="skinny_kernel", rows=64, splits=2)
+    assert plan(8192, 64, 8192) == dict(kernel="skinny_kernel", rows=64, splits=2)
+    assert plan(11008, 32, 28672) == dict(kernel="skinny_kernel", rows=128, splits=2)   # 64 rows: 172 groups, no room
+    assert plan(4096, 16, 11008) == dict(kernel="skinny_kernel", rows=32, splits=1)     # B too small to pay for it
+    assert plan(8192, 16, 16384) == dict(kernel="skinny_kernel", rows=32, splits=1)
     assert plan(65536, 64, 8192)["kernel"] == "gemm_kernel"      # from about 48k rows on the main kernel is faster
     assert plan(4096, 65, 4096)["kernel"] == "gemm_kernel"
     # fewer than 256 tiles of 512 x 128: tile and split from the cost model
@@ -169,7 +177,7 @@ def test_launch_plan_follows_the_hooks(_default_hooks):
     assert plan(11008, 16, 4096)["kernel"] == "gemm_kernel"
     _native.set_skinny_enabled(True)
     _native.set_skinny_rows(32)
-    assert plan(28672, 16, 8192) == dict(kernel="skinny_kernel", rows=32)
+    assert plan(28672, 16, 8192) == dict(kernel="skinny_kernel", rows=32, splits=1)
     _native.set_tile_config(4)
     _native.set_split_k(3)
     assert plan(8192, 8192, 8192) == dict(kernel="gemm_kernel", tile=4, splits=3, pad_b=False)

@@ -289,7 +289,7 @@ def test_one_call_entry_point_on_several_streams_keeps_the_reordered_weights_apa
 def test_split_k_kernel_large_m_row_groups(m, k, n, rows):
     """the row groups the C ABI picks for many weight rows: 64 rows at 33 ... 64 columns, 128 rows at 17 ... 32
     (partial tiles reduced in two rounds); exact on integers against the oracle"""
-    assert _native.describe_launch(m, n, k) == dict(kernel="skinny_kernel", rows=rows)
+    assert _native.describe_launch(m, n, k) == dict(kernel="skinny_kernel", rows=rows, splits=1)
     a, meta = synthetic.make_weight(m, k, seed=m + n)
     dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
     bi = synthetic.make_b(k, n, seed=n, kind="int")
@@ -326,6 +326,42 @@ def test_split_k_kernel_long_k(m, k, ns):
             assert np.array_equal(d.cpu().numpy(), exact), (n, rows, skinny)
             assert np.array_equal(y.cpu().numpy(), exact.T), (n, rows, skinny, "token-major")
     del dense
+
+
+@pytest.mark.parametrize("rows,splits", [(32, 2), (64, 3), (64, 16), (128, 4), (-1, -1)])
+@pytest.mark.parametrize("m,n,k", [(256, 16, 8192), (192, 5, 4128), (320, 32, 12320), (128, 40, 8224), (1024, 64, 16384),
+                                   (4096, 16, 16384)])
+def test_split_k_kernel_with_k_split_over_workgroups(rows, splits, m, n, k):
+    """the split-K kernel with K split over workgroups as well (partial sums + ordered reduction): forced split counts
+    that do and do not divide the chunk count, splits with fewer chunks than wavefronts, K tails, every image width,
+    beta != 0, fp16 and fp32 results, plain and token-major form with bias; the last shape splits by the plan's own
+    choice"""
+    _native.set_skinny_rows(rows)
+    _native.set_split_k(splits)
+    plan = _native.describe_launch(m, n, k)
+    assert plan["kernel"] == "skinny_kernel"
+    if (m, n, k) == (4096, 16, 16384) and splits == -1:
+        assert plan["splits"] == 4
+    a, meta = synthetic.make_weight(m, k, seed=rows + m + k + splits)
+    dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
+    bi = synthetic.make_b(k, n, seed=n, kind="int")
+    ci = synthetic.make_c(m, n, seed=n + 1, dtype=torch.float32).round()
+    exact = oracle.blas_matmul(dense, bi.numpy(), c=ci.numpy(), alpha=2.0, beta=1.0, dtype=np.float32)  # integers: exact
+    got = _run_prepared(a, meta, bi, m, n, k, c=ci, alpha=2.0, beta=1.0, out_dtype=torch.float32)
+    assert np.array_equal(got, exact)
+    plain = oracle.blas_matmul(dense, bi.numpy(), dtype=np.float32)
+    assert np.array_equal(_run_prepared(a, meta, bi, m, n, k, out_dtype=torch.float16), plain.astype(np.float16))
+    # token-major form with a bias
+    bias = synthetic.make_b(1, m, seed=n + 2, kind="int").reshape(m)
+    prep = _native.prepare(a.cuda(), meta.cuda(), m, k)
+    for y_dtype in (torch.float32, torch.float16):
+        y = torch.full((n, m), float("nan"), dtype=y_dtype, device="cuda")
+        _native.linear_prepared(prep, bi.T.contiguous().cuda(), y, m, k, bias=bias.cuda())
+        torch.cuda.synchronize()
+        want = (plain.T + bias.numpy().astype(np.float32)[None, :]).astype(np.float32 if y_dtype == torch.float32 else np.float16)
+        assert np.array_equal(y.cpu().numpy(), want), y_dtype
+    b = synthetic.make_b(k, n, seed=n + 50, kind="normal")
+    _assert_close(_run_prepared(a, meta, b, m, n, k), oracle.blas_matmul(dense, b.numpy()))
 
 
 def test_config3_split_k_is_deterministic_and_reusable():

@@ -30,12 +30,13 @@ def test_two_calls_in_a_row_second_smaller():
         hook(-1)
     _native.set_skinny_enabled(True)
     _native.set_pad_b(True)
-    # (m, n, k): K split over workgroups and a padded copy of B in the first two, a split alone in the third, no
-    # buffer at all (split-K kernel) in the last
-    shapes = ((2048, 130, 8192), (1024, 100, 8192), (512, 72, 4096), (1024, 16, 4096))
+    # (m, n, k): K split over workgroups and a padded copy of B in the first two, the split-K kernel with a K split over
+    # workgroups in the third, a split of the main kernel alone in the fourth, no buffer at all in the last
+    shapes = ((2048, 130, 8192), (1024, 100, 8192), (2048, 16, 16384), (512, 72, 4096), (1024, 16, 4096))
     plans = [_native.describe_launch(m, n, k) for (m, n, k) in shapes]
     assert plans[0]["splits"] > 1 and plans[0]["pad_b"] and plans[1]["splits"] > 1 and plans[1]["pad_b"]
-    assert plans[2]["splits"] > 1 and plans[3]["kernel"] == "skinny_kernel"
+    assert plans[2]["kernel"] == "skinny_kernel" and plans[2]["splits"] > 1   # the split-K kernel's own K split
+    assert plans[3]["splits"] > 1 and plans[4] == dict(kernel="skinny_kernel", rows=32, splits=1)
     for kind in ("int", "normal"):
         for i, (m, n, k) in enumerate(shapes):
             a, meta = synthetic.make_weight(m, k, seed=40 + i)
