@@ -39,12 +39,14 @@ def test_random_cases_match_the_oracle(seed):
                      split=int(rng.choice([-1, -1, 1, 2, 3, 5])), tile=int(rng.choice([-1, -1, -1] + list(range(15)))),
                      pad=bool(rng.random() < 0.8))
         offset = int(rng.choice([0, 0, 1, 4, 8]))  # halves: B 2, 8 or 16 bytes past a 16-byte boundary
+        static = bool(rng.random() < 0.4)          # the entry point whose buffers live in the fixed device array
         _native.set_skinny_enabled(hooks["skinny"])
         _native.set_skinny_rows(hooks["rows"])
         _native.set_split_k(hooks["split"])
         _native.set_tile_config(hooks["tile"])
         _native.set_pad_b(hooks["pad"])
-        what = f"seed {seed} case {case}: m={m} n={n} k={k} alpha={alpha} beta={beta} {out_dtype} {hooks} offset={offset}"
+        what = (f"seed {seed} case {case}: m={m} n={n} k={k} alpha={alpha} beta={beta} {out_dtype} {hooks} offset={offset} "
+                f"static={static}")
         a, meta = synthetic.make_weight(m, k, seed=int(rng.integers(1 << 30)))
         dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
         bi = synthetic.make_b(k, n, seed=case, kind="int")
@@ -57,7 +59,8 @@ def test_random_cases_match_the_oracle(seed):
         bd = storage[offset:offset + k * n].view(k, n)
         bd.copy_(bi.cuda())
         d = torch.full((m, n), float("nan"), dtype=out_dtype, device="cuda")
-        _native.matmul_prepared(prep, bd, d, m, n, k, c=ci.cuda() if beta else None, alpha=alpha, beta=beta)
+        _native.matmul_prepared(prep, bd, d, m, n, k, c=ci.cuda() if beta else None, alpha=alpha, beta=beta,
+                                static_scratch=static)
         torch.cuda.synchronize()
         assert np.array_equal(d.cpu().numpy(), want), what
         # the layer's form of the same product (tiles without a token-major variant: automatic choice)
