@@ -1171,37 +1171,54 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   // the SMFMACs of image SUB_INDEX of a chunk: steps SUB_INDEX * IMG_STEPS ... + IMG_STEPS - 1
   auto compute = [&](const AChunk (&a)[R], auto sub_tag) __attribute__((always_inline)) {
     constexpr int FIRST_STEP = decltype(sub_tag)::value * IMG_STEPS;
-    // FG fragments (4 FG transpose reads) in flight, then their SMFMACs back to back; the scheduling barriers keep
-    // the next group's reads from being hoisted (8 registers per fragment)
+    // Fragments are read in groups of FG K steps (4 FG transpose reads per column fragment) into one of two register
+    // sets: while the SMFMACs of a group run, the reads of the next group are already in flight, so only the first
+    // group of an image waits for LDS. The scheduling barriers keep later groups' reads from being hoisted as well
+    // (8 registers per fragment). Sixteen-wavefront workgroups have 128 registers per wavefront and no room for the
+    // second set: they read each group when it is due.
+    constexpr bool kAhead = NW <= 8;
     constexpr int FG = (R >= 4 || NF > 1) ? 2 : 4;
-    half16_t bfrag[FG][NF];
-    auto step = [&](auto step_tag) __attribute__((always_inline)) {
-      constexpr int STEP = decltype(step_tag)::value;
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const half8_t av = expand_signs<STEP>(a[r], one);
-#pragma unroll
-        for (int f = 0; f < NF; ++f) acc[r][f] = smfmac_step<STEP, false>(a[r], av, bfrag[STEP % FG][f], acc[r][f]);
-      }
-    };
-    auto group = [&](auto first_tag) __attribute__((always_inline)) {
-      constexpr int FIRST = decltype(first_tag)::value;  // step within the chunk
+    constexpr int GROUPS = IMG_STEPS / FG;
+    static_assert(IMG_STEPS % FG == 0 && GROUPS >= 1 && GROUPS <= 4, "whole groups of K steps per image");
+    half16_t bfrag[kAhead ? 2 : 1][FG][NF];
+    auto read_group = [&](int first_in_image, half16_t (&dst)[FG][NF]) __attribute__((always_inline)) {
 #pragma unroll
       for (int st = 0; st < FG; ++st)
 #pragma unroll
-        for (int f = 0; f < NF; ++f) bfrag[st][f] = frag(FIRST - FIRST_STEP + st, f);
-      step(std::integral_constant<int, FIRST>{});
-      step(std::integral_constant<int, FIRST + 1>{});
-      if constexpr (FG == 4) {
-        step(std::integral_constant<int, FIRST + 2>{});
-        step(std::integral_constant<int, FIRST + 3>{});
-      }
-      if (FIRST + FG < FIRST_STEP + IMG_STEPS) __builtin_amdgcn_sched_barrier(0);
+        for (int f = 0; f < NF; ++f) dst[st][f] = frag(first_in_image + st, f);
     };
-    group(std::integral_constant<int, FIRST_STEP>{});
-    if constexpr (IMG_STEPS > FG) group(std::integral_constant<int, FIRST_STEP + FG>{});
-    if constexpr (IMG_STEPS > 2 * FG) group(std::integral_constant<int, FIRST_STEP + 2 * FG>{});
-    if constexpr (IMG_STEPS > 3 * FG) group(std::integral_constant<int, FIRST_STEP + 3 * FG>{});
+    auto group = [&](auto index_tag) __attribute__((always_inline)) {
+      constexpr int G = decltype(index_tag)::value;
+      if constexpr (G < GROUPS) {
+        constexpr int FIRST = FIRST_STEP + G * FG;  // step within the chunk
+        constexpr int SET = kAhead ? (G & 1) : 0;
+        if constexpr (!kAhead) read_group(G * FG, bfrag[0]);
+        else if constexpr (G + 1 < GROUPS) read_group((G + 1) * FG, bfrag[SET ^ 1]);
+        auto step = [&](auto offset_tag) __attribute__((always_inline)) {
+          constexpr int OFFSET = decltype(offset_tag)::value;
+          if constexpr (OFFSET < FG) {
+            constexpr int STEP = FIRST + OFFSET;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+              const half8_t av = expand_signs<STEP>(a[r], one);
+#pragma unroll
+              for (int f = 0; f < NF; ++f)
+                acc[r][f] = smfmac_step<STEP, false>(a[r], av, bfrag[SET][OFFSET][f], acc[r][f]);
+            }
+          }
+        };
+        step(std::integral_constant<int, 0>{});
+        step(std::integral_constant<int, 1>{});
+        step(std::integral_constant<int, 2>{});
+        step(std::integral_constant<int, 3>{});
+        if constexpr (G + 1 < GROUPS) __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    if constexpr (kAhead) read_group(0, bfrag[0]);
+    group(std::integral_constant<int, 0>{});
+    group(std::integral_constant<int, 1>{});
+    group(std::integral_constant<int, 2>{});
+    group(std::integral_constant<int, 3>{});
   };
 
   // sixteen wavefronts leave 128 registers each: no room to hold the next image (32 registers) during the SMFMACs
