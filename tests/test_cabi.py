@@ -71,6 +71,25 @@ def test_argument_validation():
     assert "layout" in _native.last_error()
 
 
+def test_offset_limits_are_refused_with_a_message():
+    """shapes beyond the kernels' 32-bit offsets are refused before anything is launched (no GPU needed)"""
+    lib = _native.lib()
+    fake = ctypes.c_void_p(0x1000)
+    m, k = 1 << 20, 1 << 15                      # 32768 row blocks x 128 chunks x 1536 bytes = 6 GiB of prepared operand
+    assert _native.prepared_bytes(m, k) >= 1 << 32
+    assert lib.onebit_sparse_matmul_prepared(fake, fake, fake, fake, m, 128, k, 1.0, 0.0, 0, 0, None) == 1
+    assert "4 GiB" in _native.last_error()
+    assert lib.onebit_sparse_linear_prepared(fake, fake, None, fake, 128, m, k, 1, 1, None) == 1
+    assert "4 GiB" in _native.last_error()
+    assert lib.onebit_sparse_matmul_prepared_static(fake, fake, fake, fake, m, 128, k, 1.0, 0.0, 0, 0, None) in (1, 2)
+    # the token-major form addresses a tile's token rows with 32-bit offsets: k is limited
+    assert lib.onebit_sparse_linear_prepared(fake, fake, None, fake, 128, 64, 1 << 23, 1, 1, None) == 1
+    assert "token-major" in _native.last_error()
+    # x must be 16-byte aligned
+    assert lib.onebit_sparse_linear_prepared(fake, ctypes.c_void_p(0x1008), None, fake, 8, 64, 64, 1, 1, None) == 1
+    assert "aligned" in _native.last_error()
+
+
 @pytest.mark.skipif(torch.cuda.is_available(), reason="needs a host without a GPU (pointers are fake)")
 def test_no_device_is_reported_not_fatal():
     lib = _native.lib()
