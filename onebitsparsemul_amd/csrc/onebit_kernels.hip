@@ -310,6 +310,31 @@ __device__ __forceinline__ void expand_frags(const AChunk (&a)[FM], uint32_t one
   for (int fm = 0; fm < FM; ++fm) av[fm] = expand_signs<STEP>(a[fm], one);
 }
 
+// Sign expansion that stays where it is written: the optimizer otherwise sinks it past the stage's barrier to the
+// block of its first use.
+template <int STEP>
+__device__ __forceinline__ half8_t expand_signs_here(const AChunk& a, uint32_t packed_one) {
+  half8_t v = expand_signs<STEP>(a, packed_one);
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
+// One packed register (kept values 2p, 2p+1 of K step STEP) of the same expansion, also kept where it is written.
+template <int STEP>
+__device__ __forceinline__ uint32_t expand_sign_register(const AChunk& a, uint32_t packed_one, int p) {
+  const uint32_t w = STEP < 4 ? a.sign.x : a.sign.y;
+  uint32_t v = ((w << (4 * (STEP % 4) + p)) & 0x80008000u) | packed_one;
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
+// Same, kept where it is written (see expand_signs_here).
+template <int STEP, int FM>
+__device__ __forceinline__ void expand_frags_here(const AChunk (&a)[FM], uint32_t one, half8_t (&av)[FM]) {
+#pragma unroll
+  for (int fm = 0; fm < FM; ++fm) av[fm] = expand_signs_here<STEP>(a[fm], one);
+}
+
 template <int STEP, int FM, int FN>
 __device__ __forceinline__ void mfma_frags(const AChunk (&a)[FM], const half8_t (&av)[FM], const half16_t (&bv)[FN],
                                            float16_t (&acc)[FM][FN]) {
@@ -319,6 +344,44 @@ __device__ __forceinline__ void mfma_frags(const AChunk (&a)[FM], const half8_t 
   for (int fm = 0; fm < FM; ++fm)
 #pragma unroll
     for (int fn = 0; fn < FN; ++fn) acc[fm][fn] = smfmac_step<STEP, (FM * FN > 8)>(a[fm], av[fm], bv[fn], acc[fm][fn]);
+}
+
+// One piece of the B fragments of a K step: piece r of the row-major image is transpose read q = r % 4 of fragment
+// r / 4, piece r of the token-major image is 16-byte read h = r % 2 of fragment r / 2.
+template <int BN>
+__device__ __forceinline__ void load_b_piece(const char* stage_lds, int ks, int r, u32x8_t* bv, const int* frag_off,
+                                             int lane_row_off) {
+  const int fn = r >> 2, q = r & 3;
+  const int row_const = ks * 32 + 4 * (q & 1) + 16 * (q >> 1);
+  const u32x2_t t = lds_read_tr16(stage_lds + lane_row_off + row_const * (BN * 2) + frag_off[fn]);
+  bv[fn][2 * q] = t.x;
+  bv[fn][2 * q + 1] = t.y;
+}
+
+__device__ __forceinline__ void load_b_piece_tokens(const char* wave_lds, int ks, int r, u32x8_t* bv,
+                                                    const int* piece_off) {
+  const int fn = r >> 1, h = r & 1;
+  const u32x4_t t = *reinterpret_cast<const u32x4_t*>(wave_lds + piece_off[2 * ks + h] + fn * (32 * kStageK * 2));
+  bv[fn][4 * h] = t.x; bv[fn][4 * h + 1] = t.y; bv[fn][4 * h + 2] = t.z; bv[fn][4 * h + 3] = t.w;
+}
+
+// The SMFMACs of one K step of a one-wavefront-per-SIMD tile with the fetch work of the next step placed between
+// them by hand: fetch(slot) runs right behind SMFMAC number `slot`. Such a tile has no second wavefront on its SIMD to
+// fill the matrix pipe while this one reads fragments and expands signs, and the compiler keeps the inline-assembly
+// SMFMACs in one block, so the interleaving is written out and fenced.
+template <int STEP, bool PINNED, int FM, int FN, class Fetch>
+__device__ __forceinline__ void mfma_frags_fused(const AChunk (&a)[FM], const u32x4_t (&av)[FM], const u32x8_t (&bv)[FN],
+                                                 float16_t (&acc)[FM][FN], Fetch&& fetch) {
+#pragma unroll
+  for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+    for (int fn = 0; fn < FN; ++fn) {
+      acc[fm][fn] = smfmac_step<STEP, PINNED>(a[fm], __builtin_bit_cast(half8_t, av[fm]),
+                                              __builtin_bit_cast(half16_t, bv[fn]), acc[fm][fn]);
+      __builtin_amdgcn_sched_barrier(0);
+      fetch(fm * FN + fn);
+      __builtin_amdgcn_sched_barrier(0);
+    }
 }
 
 // Source of zeros for the asynchronous copies of B rows at or past K.
@@ -452,6 +515,13 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
       b_stage += stage_stride;
       next_k0 += kStageK;
     };
+    // the same for a stage that the caller knows to lie inside K: no branch, so that the K loop's body stays one block
+    auto issue_b_full = [&](int ring) {
+#pragma unroll
+      for (int i = 0; i < NL; ++i) lds_dma16_base(b_stage, b_off[i], lds_dst[i] + ring * TS::STAGE_BYTES);
+      b_stage += stage_stride;
+      next_k0 += kStageK;
+    };
 
     // ---- asynchronous copy pattern for A: the workgroup's BM/32 prepared blocks of one K chunk ----
     // LDS image = the blocks back to back; NA copies of 1 KiB per wavefront (the tail past the last block
@@ -475,80 +545,112 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
     }
     const char* a_chunk = reinterpret_cast<const char*>(p.prep) + (size_t)chunk_begin * kBlockBytes;  // advances one K chunk per copy
     int next_chunk = chunk_begin;
+    auto advance_a = [&]() {
+      if (next_chunk + 1 < chunks) a_chunk += kBlockBytes;  // past the last chunk the last one is copied again
+      ++next_chunk;
+    };
     auto issue_a = [&]() {
 #pragma unroll
       for (int j = 0; j < NA; ++j) lds_dma16_base(a_chunk, a_off[j], a_dst[j]);
-      if (next_chunk + 1 < chunks) a_chunk += kBlockBytes;  // past the last chunk the last one is copied again
-      ++next_chunk;
+      advance_a();
     };
     const char* a_frag_lds[FM];
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm) a_frag_lds[fm] = a_lds + (wm * FM + fm) * kBlockBytes;
 
     if constexpr (KG == 1) {
-      // Software pipeline. One K step (32 wide) is one scheduling region in which the SMFMACs of the step run
-      // while the B fragments and the expanded A of the next step are fetched. The workgroup barrier sits in the
-      // middle of each stage s: it publishes stage s+1 (read right after it) and frees the ring slot of stage s
-      // (all of its reads were issued in the first half), into which stage s+4 is then copied.
-      // Request order: A(0) B(0) B(1) B(2) B(3) | chunk c: mid s0: A(c+1) B(4c+4)  mid s1: B(4c+5)
-      //                                                     mid s2: B(4c+6)        mid s3: B(4c+7)
+      // Same stages, barriers, request order and wait counts as the pipeline below, with the order of the instructions
+      // inside each K-step region written out: behind SMFMAC number `slot` of the step comes that slot's share of the
+      // fetch work for the next step (fragment reads in the first half of the slots, two sign-expansion instructions per
+      // register spread evenly), and after a barrier the first SMFMAC precedes the copies.
       issue_a();
 #pragma unroll
       for (int s = 0; s < kStages; ++s) issue_b(s);
 
-      AChunk a_cur[FM];
-      half16_t bv0[FN], bv1[FN];
-      half8_t av0[FM], av1[FM];
+      constexpr bool PINNED = FM * FN > 8;
+      constexpr int SLOTS = FM * FN;
+      constexpr int PIECES = TOKENS ? 2 * FN : 4 * FN;
+      constexpr int PPS = (2 * PIECES + SLOTS - 1) / SLOTS > 1 ? (2 * PIECES + SLOTS - 1) / SLOTS : 1;  // pieces per slot
+      AChunk a_cur[FM], a_next[FM];
+      u32x8_t bv0[FN], bv1[FN];
+      u32x4_t av0[FM], av1[FM];
+      auto read_piece = [&](int ring_slot, int ks, int r, u32x8_t* bv) __attribute__((always_inline)) {
+        if constexpr (TOKENS) load_b_piece_tokens(wave_image + ring_slot * TS::STAGE_BYTES, ks, r, bv, piece_off);
+        else load_b_piece<BN>(smem + ring_slot * TS::STAGE_BYTES, ks, r, bv, frag_off, lane_row_off);
+      };
       wait_vmcnt<3 * NL>();  // A(0) and B(0) have landed
       __builtin_amdgcn_s_barrier();
 #pragma unroll
       for (int fm = 0; fm < FM; ++fm) a_cur[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);
-      read_frags(0, 0, bv0);
-      expand_frags<0>(a_cur, one, av0);
+#pragma unroll
+      for (int r = 0; r < PIECES; ++r) read_piece(0, 0, r, bv0);
+#pragma unroll
+      for (int g = 0; g < 4 * FM; ++g) av0[g / 4][g % 4] = expand_sign_register<0>(a_cur[g / 4], one, g % 4);
 
-#define ONEBIT_STAGE(S, WAITCNT, ISSUE_A)                                                                        \
+// the fetch work behind SMFMAC `slot`: pieces of the fragments of (RING, KS) into BV, registers of step FILL_STEP of A_SRC into AV
+#define ONEBIT_FETCH_SLOT(RING, KS, BV, FILL_STEP, A_SRC, AV)                                                      \
+          _Pragma("unroll") for (int r = 0; r < PIECES; ++r)                                                        \
+            if (r / PPS == slot) read_piece((RING), (KS), r, BV);                                                   \
+          _Pragma("unroll") for (int g = 0; g < 4 * FM; ++g)                                                        \
+            if (g * FN / 4 == slot) AV[g / 4][g % 4] = expand_sign_register<(FILL_STEP)>(A_SRC[g / 4], one, g % 4);
+#define ONEBIT_FUSED_STAGE(S, WAITCNT, ISSUE_A)                                                                  \
       {                                                                                                            \
-        read_frags((S), 1, bv1);                                                                                   \
-        expand_frags<2 * (S) + 1>(a_cur, one, av1);                                                                \
-        mfma_frags<2 * (S)>(a_cur, av0, bv0, acc);                                                                 \
-        __builtin_amdgcn_sched_barrier(0); /* keep the step's work inside its region */                           \
-        wait_vmcnt_lgkm0<(WAITCNT)>(); /* copies of stage S+1 landed; this wavefront's reads of stage S returned */      \
-        __builtin_amdgcn_s_barrier();                                                                              \
-        if (ISSUE_A) issue_a();                                                                                    \
-        issue_b(S);                                                                                                \
-        read_frags(((S) + 1) % kStages, 0, bv0);                                                                   \
+        mfma_frags_fused<2 * (S), PINNED>(a_cur, av0, bv0, acc, [&](int slot) __attribute__((always_inline)) {     \
+          ONEBIT_FETCH_SLOT((S), 1, bv1, 2 * (S) + 1, a_cur, av1)                                                  \
+        });                                                                                                        \
+        wait_vmcnt_lgkm0<(WAITCNT)>(); /* copies of stage S+1 landed; this wavefront's reads of stage S returned */ \
+        __builtin_amdgcn_s_barrier();                                                                   \
+        if constexpr ((S) == kStages - 1) {                                                                        \
+          /* the next chunk of A is readable after this stage's barrier */                                         \
+          _Pragma("unroll") for (int fm = 0; fm < FM; ++fm) a_next[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);   \
+          __builtin_amdgcn_sched_barrier(0);                                                                       \
+        }                                                                                                          \
+        mfma_frags_fused<2 * (S) + 1, PINNED>(a_cur, av1, bv1, acc, [&](int slot) __attribute__((always_inline)) { \
+          if constexpr (FULL) {                                                                                    \
+            /* copy c of the stage (A first, same request order) behind SMFMAC c / CPS */                          \
+            constexpr int COPIES = ((ISSUE_A) ? NA : 0) + NL, CPS = (COPIES + SLOTS - 1) / SLOTS;                  \
+            _Pragma("unroll") for (int c = 0; c < COPIES; ++c)                                                     \
+              if (c / CPS == slot) {                                                                               \
+                const int i = c - ((ISSUE_A) ? NA : 0);                                                            \
+                if (i < 0) lds_dma16_base(a_chunk, a_off[c], a_dst[c]);                                            \
+                else lds_dma16_base(b_stage, b_off[i], lds_dst[i] + (S) * TS::STAGE_BYTES);                        \
+              }                                                                                                    \
+            if (slot == (COPIES - 1) / CPS) {                                                                      \
+              if (ISSUE_A) advance_a();                                                                            \
+              b_stage += stage_stride;                                                                             \
+              next_k0 += kStageK;                                                                                  \
+            }                                                                                                      \
+            __builtin_amdgcn_sched_barrier(0);                                                                     \
+          } else if (slot == 0) {                                                                                  \
+            if (ISSUE_A) issue_a();                                                                                \
+            issue_b(S);                                                                                            \
+            __builtin_amdgcn_sched_barrier(0);                                                                     \
+          }                                                                                                        \
+          if constexpr ((S) < kStages - 1) {                                                                       \
+            ONEBIT_FETCH_SLOT((S) + 1, 0, bv0, 2 * (S) + 2, a_cur, av0)                                            \
+          } else {                                                                                                 \
+            ONEBIT_FETCH_SLOT(0, 0, bv0, 0, a_next, av0)                                                           \
+          }                                                                                                        \
+        });                                                                                                        \
+        if constexpr ((S) == kStages - 1) {                                                                        \
+          _Pragma("unroll") for (int fm = 0; fm < FM; ++fm) a_cur[fm] = a_next[fm];                                \
+        }                                                                                                          \
       }
 
-      for (int kc = chunk_begin; kc < chunk_end; ++kc) {
-        // mid stage 0: waits for B(4c+1); newer requests: B(4c+2), B(4c+3)
-        ONEBIT_STAGE(0, 2 * NL, true)
-        expand_frags<2>(a_cur, one, av0);
-        mfma_frags<1>(a_cur, av1, bv1, acc);
-        __builtin_amdgcn_sched_barrier(0);
-        // mid stage 1: waits for B(4c+2); newer: B(4c+3), A(c+1), B(4c+4)
-        ONEBIT_STAGE(1, 2 * NL + NA, false)
-        expand_frags<4>(a_cur, one, av0);
-        mfma_frags<3>(a_cur, av1, bv1, acc);
-        __builtin_amdgcn_sched_barrier(0);
-        // mid stage 2: waits for B(4c+3); newer: A(c+1), B(4c+4), B(4c+5)
-        ONEBIT_STAGE(2, 2 * NL + NA, false)
-        expand_frags<6>(a_cur, one, av0);
-        mfma_frags<5>(a_cur, av1, bv1, acc);
-        __builtin_amdgcn_sched_barrier(0);
-        // mid stage 3: waits for B(4c+4), which is newer than A(c+1): the next chunk of A is readable after it
-        ONEBIT_STAGE(3, 2 * NL, false)
-        {
-          AChunk a_next[FM];
-#pragma unroll
-          for (int fm = 0; fm < FM; ++fm) a_next[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);
-          expand_frags<0>(a_next, one, av0);
-          mfma_frags<7>(a_cur, av1, bv1, acc);
-#pragma unroll
-          for (int fm = 0; fm < FM; ++fm) a_cur[fm] = a_next[fm];
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-#undef ONEBIT_STAGE
+      auto chunk_body = [&](auto full_tag) __attribute__((always_inline)) {
+        constexpr bool FULL = decltype(full_tag)::value;  // the four stages copied during this chunk lie inside K
+        ONEBIT_FUSED_STAGE(0, 2 * NL, true)        // waits for B(4c+1); newer requests: B(4c+2), B(4c+3)
+        ONEBIT_FUSED_STAGE(1, 2 * NL + NA, false)  // waits for B(4c+2); newer: B(4c+3), A(c+1), B(4c+4)
+        ONEBIT_FUSED_STAGE(2, 2 * NL + NA, false)  // waits for B(4c+3); newer: A(c+1), B(4c+4), B(4c+5)
+        ONEBIT_FUSED_STAGE(3, 2 * NL, false)       // waits for B(4c+4), which is newer than A(c+1)
+      };
+      // chunk kc copies the stages of chunk kc + 1: they are whole while (kc + 2) * 256 <= K
+      int kc = chunk_begin;
+      const int full_end = p.k / kChunkK - 1 < chunk_end ? p.k / kChunkK - 1 : chunk_end;
+      for (; kc < full_end; ++kc) chunk_body(std::true_type{});
+      for (; kc < chunk_end; ++kc) chunk_body(std::false_type{});
+#undef ONEBIT_FUSED_STAGE
+#undef ONEBIT_FETCH_SLOT
       wait_vmcnt<0>();  // drain the copies issued past the end before the LDS is released
     } else {
       // Two K groups: this wavefront multiplies K step KGV of every stage. One barrier per stage: before it the
@@ -578,12 +680,12 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
           issue_b(S);                                                                                            \
           read_frags(((S) + 1) % kStages, KGV, BV_NEXT);                                                         \
           if constexpr ((S) < kStages - 1) {                                                                     \
-            expand_frags<2 * ((S) + 1) + KGV>(a_cur, one, AV_NEXT);                                              \
+            expand_frags_here<2 * ((S) + 1) + KGV>(a_cur, one, AV_NEXT);                                              \
             mfma_frags<2 * (S) + KGV>(a_cur, AV, BV, acc);                                                       \
           } else {                                                                                               \
             AChunk a_next[FM];                                                                                   \
             _Pragma("unroll") for (int fm = 0; fm < FM; ++fm) a_next[fm] = load_a_chunk_lds(a_frag_lds[fm], lane); \
-            expand_frags<KGV>(a_next, one, AV_NEXT);                                                             \
+            expand_frags_here<KGV>(a_next, one, AV_NEXT);                                                           \
             mfma_frags<2 * (S) + KGV>(a_cur, AV, BV, acc);                                                       \
             _Pragma("unroll") for (int fm = 0; fm < FM; ++fm) a_cur[fm] = a_next[fm];                            \
           }                                                                                                      \
