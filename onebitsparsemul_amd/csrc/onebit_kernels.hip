@@ -259,25 +259,7 @@ __device__ __forceinline__ void compute_stage(const char* stage_lds, const AChun
   }
 }
 
-// ---- software-pipelined building blocks of the asynchronous-copy main loop -------------------------
-// B fragments of one 32-wide K step (ks = 0/1 inside a 64-row stage image).
-template <int FN, int BN>
-__device__ __forceinline__ void load_b_frags(const char* stage_lds, int ks, half16_t (&bv)[FN], const int (&frag_off)[FN],
-                                             int lane_row_off) {
-#pragma unroll
-  for (int fn = 0; fn < FN; ++fn) {
-    u32x8_t raw;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int row_const = ks * 32 + 4 * (q & 1) + 16 * (q >> 1);
-      const u32x2_t t = lds_read_tr16(stage_lds + lane_row_off + row_const * (BN * 2) + frag_off[fn]);
-      raw[2 * q] = t.x;
-      raw[2 * q + 1] = t.y;
-    }
-    bv[fn] = __builtin_bit_cast(half16_t, raw);
-  }
-}
-
+// ---- building blocks of the asynchronous-copy main loop ----------------------------------------------
 // Token-major stage image (linear-layer form): row t = the stage's 64 K values of token t (128 bytes, eight 16-byte
 // pieces, piece p stored at position p ^ token_swizzle(t)). The operand of K step ks is pieces 4 ks + gb and 4 ks + 2 + gb of
 // the lane's token: two plain 16-byte reads at the precomputed lane offsets piece_off[2 ks + h].
@@ -289,61 +271,15 @@ __device__ __forceinline__ constexpr int token_swizzle(int token) {
   return ROW_BYTES >= 256 ? (token & 15) : ((token >> 1) & 7);
 }
 
-template <int FN>
-__device__ __forceinline__ void load_b_frags_tokens(const char* wave_lds, int ks, half16_t (&bv)[FN],
-                                                    const int (&piece_off)[4]) {
-#pragma unroll
-  for (int fn = 0; fn < FN; ++fn) {
-    u32x8_t raw;
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const u32x4_t t = *reinterpret_cast<const u32x4_t*>(wave_lds + piece_off[2 * ks + h] + fn * (32 * kStageK * 2));
-      raw[4 * h] = t.x; raw[4 * h + 1] = t.y; raw[4 * h + 2] = t.z; raw[4 * h + 3] = t.w;
-    }
-    bv[fn] = __builtin_bit_cast(half16_t, raw);
-  }
-}
-
-template <int STEP, int FM>
-__device__ __forceinline__ void expand_frags(const AChunk (&a)[FM], uint32_t one, half8_t (&av)[FM]) {
-#pragma unroll
-  for (int fm = 0; fm < FM; ++fm) av[fm] = expand_signs<STEP>(a[fm], one);
-}
-
-// Sign expansion that stays where it is written: the optimizer otherwise sinks it past the stage's barrier to the
-// block of its first use.
-template <int STEP>
-__device__ __forceinline__ half8_t expand_signs_here(const AChunk& a, uint32_t packed_one) {
-  half8_t v = expand_signs<STEP>(a, packed_one);
-  asm volatile("" : "+v"(v));
-  return v;
-}
-
-// One packed register (kept values 2p, 2p+1 of K step STEP) of the same expansion, also kept where it is written.
+// One packed register (kept values 2p, 2p+1 of K step STEP) of expand_signs. The empty volatile statement keeps the two
+// instructions where they are written: the optimizer otherwise sinks them past the stage's barrier to the block of their
+// first use.
 template <int STEP>
 __device__ __forceinline__ uint32_t expand_sign_register(const AChunk& a, uint32_t packed_one, int p) {
   const uint32_t w = STEP < 4 ? a.sign.x : a.sign.y;
   uint32_t v = ((w << (4 * (STEP % 4) + p)) & 0x80008000u) | packed_one;
   asm volatile("" : "+v"(v));
   return v;
-}
-
-// Same, kept where it is written (see expand_signs_here).
-template <int STEP, int FM>
-__device__ __forceinline__ void expand_frags_here(const AChunk (&a)[FM], uint32_t one, half8_t (&av)[FM]) {
-#pragma unroll
-  for (int fm = 0; fm < FM; ++fm) av[fm] = expand_signs_here<STEP>(a[fm], one);
-}
-
-template <int STEP, int FM, int FN>
-__device__ __forceinline__ void mfma_frags(const AChunk (&a)[FM], const half8_t (&av)[FM], const half16_t (&bv)[FN],
-                                           float16_t (&acc)[FM][FN]) {
-  // pinned accumulators only for the one-wavefront-per-SIMD tiles: the two-per-SIMD tiles have 128 vector
-  // registers left beside their 128 accumulators, which the pinned form overflows
-#pragma unroll
-  for (int fm = 0; fm < FM; ++fm)
-#pragma unroll
-    for (int fn = 0; fn < FN; ++fn) acc[fm][fn] = smfmac_step<STEP, (FM * FN > 8)>(a[fm], av[fm], bv[fn], acc[fm][fn]);
 }
 
 // One piece of the B fragments of a K step: piece r of the row-major image is transpose read q = r % 4 of fragment
@@ -365,10 +301,9 @@ __device__ __forceinline__ void load_b_piece_tokens(const char* wave_lds, int ks
   bv[fn][4 * h] = t.x; bv[fn][4 * h + 1] = t.y; bv[fn][4 * h + 2] = t.z; bv[fn][4 * h + 3] = t.w;
 }
 
-// The SMFMACs of one K step of a one-wavefront-per-SIMD tile with the fetch work of the next step placed between
-// them by hand: fetch(slot) runs right behind SMFMAC number `slot`. Such a tile has no second wavefront on its SIMD to
-// fill the matrix pipe while this one reads fragments and expands signs, and the compiler keeps the inline-assembly
-// SMFMACs in one block, so the interleaving is written out and fenced.
+// The SMFMACs of one K step with the fetch work for the next step placed between them by hand: fetch(slot) runs right
+// behind SMFMAC number `slot`, and scheduling fences keep it there (the compiler would otherwise keep the
+// inline-assembly SMFMACs of the one-wavefront-per-SIMD tiles in one block, and order the rest as it likes).
 template <int STEP, bool PINNED, int FM, int FN, class Fetch>
 __device__ __forceinline__ void mfma_frags_fused(const AChunk (&a)[FM], const u32x4_t (&av)[FM], const u32x8_t (&bv)[FN],
                                                  float16_t (&acc)[FM][FN], Fetch&& fetch) {
@@ -439,10 +374,6 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
     for (int j = 0; j < 4; ++j) piece_off[j] = base ^ ((4 * (j >> 1) + 2 * (j & 1)) << 4);
   }
   const char* const wave_image = smem + wn * FN * (32 * kStageK * 2);  // first token row of this wavefront in stage 0
-  auto read_frags = [&](int ring_slot, int ks, half16_t (&bv)[FN]) __attribute__((always_inline)) {
-    if constexpr (TOKENS) load_b_frags_tokens<FN>(wave_image + ring_slot * TS::STAGE_BYTES, ks, bv, piece_off);
-    else load_b_frags<FN, BN>(smem + ring_slot * TS::STAGE_BYTES, ks, bv, frag_off, lane_row_off);
-  };
 
   const uint32_t one = packed_one_in_vgpr();
   float16_t acc[FM][FN];
@@ -558,56 +489,36 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm) a_frag_lds[fm] = a_lds + (wm * FM + fm) * kBlockBytes;
 
-    if constexpr (KG == 1) {
-      // Same stages, barriers, request order and wait counts as the pipeline below, with the order of the instructions
-      // inside each K-step region written out: behind SMFMAC number `slot` of the step comes that slot's share of the
-      // fetch work for the next step (fragment reads in the first half of the slots, two sign-expansion instructions per
-      // register spread evenly), and after a barrier the first SMFMAC precedes the copies.
-      issue_a();
-#pragma unroll
-      for (int s = 0; s < kStages; ++s) issue_b(s);
-
-      constexpr bool PINNED = FM * FN > 8;
-      constexpr int SLOTS = FM * FN;
-      constexpr int PIECES = TOKENS ? 2 * FN : 4 * FN;
-      constexpr int PPS = (2 * PIECES + SLOTS - 1) / SLOTS > 1 ? (2 * PIECES + SLOTS - 1) / SLOTS : 1;  // pieces per slot
-      AChunk a_cur[FM], a_next[FM];
-      u32x8_t bv0[FN], bv1[FN];
-      u32x4_t av0[FM], av1[FM];
-      auto read_piece = [&](int ring_slot, int ks, int r, u32x8_t* bv) __attribute__((always_inline)) {
-        if constexpr (TOKENS) load_b_piece_tokens(wave_image + ring_slot * TS::STAGE_BYTES, ks, r, bv, piece_off);
-        else load_b_piece<BN>(smem + ring_slot * TS::STAGE_BYTES, ks, r, bv, frag_off, lane_row_off);
-      };
-      wait_vmcnt<3 * NL>();  // A(0) and B(0) have landed
-      __builtin_amdgcn_s_barrier();
-#pragma unroll
-      for (int fm = 0; fm < FM; ++fm) a_cur[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);
-#pragma unroll
-      for (int r = 0; r < PIECES; ++r) read_piece(0, 0, r, bv0);
-#pragma unroll
-      for (int g = 0; g < 4 * FM; ++g) av0[g / 4][g % 4] = expand_sign_register<0>(a_cur[g / 4], one, g % 4);
-
+    // ---- the K loop ------------------------------------------------------------------------------------
+    // Software pipeline over a ring of four 64-row stages of B (and one K chunk of A) in LDS. The SMFMACs of one K step
+    // run while the B fragments and the expanded signs of the next step this wavefront multiplies are fetched; one
+    // workgroup barrier per stage publishes the next stage and frees the ring slot of the one whose reads have all been
+    // issued, into which the stage four ahead is then copied.
+    // Request order: A(0) B(0) B(1) B(2) B(3) | chunk c: stage 0: A(c+1) B(4c+4)  stage 1: B(4c+5)
+    //                                                     stage 2: B(4c+6)        stage 3: B(4c+7)
+    // The order of the instructions inside each K-step region is written out and fenced: behind SMFMAC number `slot` of
+    // the step comes that slot's share of the fetch work (fragment reads in the first half of the slots, the two
+    // instructions per sign register spread evenly, the copies one by one), so that the two wavefronts of a SIMD, which
+    // leave every barrier in lock-step, alternate on the matrix pipe instead of both fetching first; left to itself the
+    // optimizer sinks the sign expansion past the barrier to the block of its first use.
+    constexpr bool PINNED = FM * FN > 8;
+    constexpr int SLOTS = FM * FN;
+    constexpr int PIECES = TOKENS ? 2 * FN : 4 * FN;
+    constexpr int PPS = (2 * PIECES + SLOTS - 1) / SLOTS > 1 ? (2 * PIECES + SLOTS - 1) / SLOTS : 1;  // pieces per slot
+    auto read_piece = [&](int ring_slot, int ks, int r, u32x8_t* bv) __attribute__((always_inline)) {
+      if constexpr (TOKENS) load_b_piece_tokens(wave_image + ring_slot * TS::STAGE_BYTES, ks, r, bv, piece_off);
+      else load_b_piece<BN>(smem + ring_slot * TS::STAGE_BYTES, ks, r, bv, frag_off, lane_row_off);
+    };
 // the fetch work behind SMFMAC `slot`: pieces of the fragments of (RING, KS) into BV, registers of step FILL_STEP of A_SRC into AV
 #define ONEBIT_FETCH_SLOT(RING, KS, BV, FILL_STEP, A_SRC, AV)                                                      \
           _Pragma("unroll") for (int r = 0; r < PIECES; ++r)                                                        \
             if (r / PPS == slot) read_piece((RING), (KS), r, BV);                                                   \
           _Pragma("unroll") for (int g = 0; g < 4 * FM; ++g)                                                        \
             if (g * FN / 4 == slot) AV[g / 4][g % 4] = expand_sign_register<(FILL_STEP)>(A_SRC[g / 4], one, g % 4);
-#define ONEBIT_FUSED_STAGE(S, WAITCNT, ISSUE_A)                                                                  \
-      {                                                                                                            \
-        mfma_frags_fused<2 * (S), PINNED>(a_cur, av0, bv0, acc, [&](int slot) __attribute__((always_inline)) {     \
-          ONEBIT_FETCH_SLOT((S), 1, bv1, 2 * (S) + 1, a_cur, av1)                                                  \
-        });                                                                                                        \
-        wait_vmcnt_lgkm0<(WAITCNT)>(); /* copies of stage S+1 landed; this wavefront's reads of stage S returned */ \
-        __builtin_amdgcn_s_barrier();                                                                   \
-        if constexpr ((S) == kStages - 1) {                                                                        \
-          /* the next chunk of A is readable after this stage's barrier */                                         \
-          _Pragma("unroll") for (int fm = 0; fm < FM; ++fm) a_next[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);   \
-          __builtin_amdgcn_sched_barrier(0);                                                                       \
-        }                                                                                                          \
-        mfma_frags_fused<2 * (S) + 1, PINNED>(a_cur, av1, bv1, acc, [&](int slot) __attribute__((always_inline)) { \
+// the copies of stage S + 4 (and of the next chunk of A) behind SMFMAC `slot`: one by one when the stage is known to lie
+// inside K (A first, same request order), else all behind the first SMFMAC through the general, branching form
+#define ONEBIT_COPY_SLOT(S, ISSUE_A)                                                                               \
           if constexpr (FULL) {                                                                                    \
-            /* copy c of the stage (A first, same request order) behind SMFMAC c / CPS */                          \
             constexpr int COPIES = ((ISSUE_A) ? NA : 0) + NL, CPS = (COPIES + SLOTS - 1) / SLOTS;                  \
             _Pragma("unroll") for (int c = 0; c < COPIES; ++c)                                                     \
               if (c / CPS == slot) {                                                                               \
@@ -625,7 +536,43 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
             if (ISSUE_A) issue_a();                                                                                \
             issue_b(S);                                                                                            \
             __builtin_amdgcn_sched_barrier(0);                                                                     \
-          }                                                                                                        \
+          }
+    // chunk kc copies the stages of chunk kc + 1: they are whole while (kc + 2) * 256 <= K
+    const int full_end = p.k / kChunkK - 1 < chunk_end ? p.k / kChunkK - 1 : chunk_end;
+
+    if constexpr (KG == 1) {
+      // The barrier sits in the middle of each stage s: it publishes stage s+1 (read right after it) and frees the ring
+      // slot of stage s (all of its reads were issued in the first half).
+      issue_a();
+#pragma unroll
+      for (int s = 0; s < kStages; ++s) issue_b(s);
+
+      AChunk a_cur[FM], a_next[FM];
+      u32x8_t bv0[FN], bv1[FN];
+      u32x4_t av0[FM], av1[FM];
+      wait_vmcnt<3 * NL>();  // A(0) and B(0) have landed
+      __builtin_amdgcn_s_barrier();
+#pragma unroll
+      for (int fm = 0; fm < FM; ++fm) a_cur[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);
+#pragma unroll
+      for (int r = 0; r < PIECES; ++r) read_piece(0, 0, r, bv0);
+#pragma unroll
+      for (int g = 0; g < 4 * FM; ++g) av0[g / 4][g % 4] = expand_sign_register<0>(a_cur[g / 4], one, g % 4);
+
+#define ONEBIT_FUSED_STAGE(S, WAITCNT, ISSUE_A)                                                                  \
+      {                                                                                                            \
+        mfma_frags_fused<2 * (S), PINNED>(a_cur, av0, bv0, acc, [&](int slot) __attribute__((always_inline)) {     \
+          ONEBIT_FETCH_SLOT((S), 1, bv1, 2 * (S) + 1, a_cur, av1)                                                  \
+        });                                                                                                        \
+        wait_vmcnt_lgkm0<(WAITCNT)>(); /* copies of stage S+1 landed; this wavefront's reads of stage S returned */ \
+        __builtin_amdgcn_s_barrier();                                                                              \
+        if constexpr ((S) == kStages - 1) {                                                                        \
+          /* the next chunk of A is readable after this stage's barrier */                                         \
+          _Pragma("unroll") for (int fm = 0; fm < FM; ++fm) a_next[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);   \
+          __builtin_amdgcn_sched_barrier(0);                                                                       \
+        }                                                                                                          \
+        mfma_frags_fused<2 * (S) + 1, PINNED>(a_cur, av1, bv1, acc, [&](int slot) __attribute__((always_inline)) { \
+          ONEBIT_COPY_SLOT(S, ISSUE_A)                                                                             \
           if constexpr ((S) < kStages - 1) {                                                                       \
             ONEBIT_FETCH_SLOT((S) + 1, 0, bv0, 2 * (S) + 2, a_cur, av0)                                            \
           } else {                                                                                                 \
@@ -644,64 +591,69 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
         ONEBIT_FUSED_STAGE(2, 2 * NL + NA, false)  // waits for B(4c+3); newer: A(c+1), B(4c+4), B(4c+5)
         ONEBIT_FUSED_STAGE(3, 2 * NL, false)       // waits for B(4c+4), which is newer than A(c+1)
       };
-      // chunk kc copies the stages of chunk kc + 1: they are whole while (kc + 2) * 256 <= K
       int kc = chunk_begin;
-      const int full_end = p.k / kChunkK - 1 < chunk_end ? p.k / kChunkK - 1 : chunk_end;
       for (; kc < full_end; ++kc) chunk_body(std::true_type{});
       for (; kc < chunk_end; ++kc) chunk_body(std::false_type{});
 #undef ONEBIT_FUSED_STAGE
-#undef ONEBIT_FETCH_SLOT
       wait_vmcnt<0>();  // drain the copies issued past the end before the LDS is released
     } else {
       // Two K groups: this wavefront multiplies K step KGV of every stage. One barrier per stage: before it the
       // wavefront waits for its fragments of stage S (read during stage S - 1) and for the copies of stage S + 1; after
-      // it the ring slot of stage S is free for stage S + 4 and stage S + 1 is readable. The fragments and the
-      // expanded signs of the next stage are fetched while the SMFMACs of this one run. Same request order and
-      // wait counts as the one-group pipeline.
+      // it the ring slot of stage S is free for stage S + 4 and stage S + 1 is readable. Same request order and wait
+      // counts as the one-group pipeline.
       auto run = [&](auto group_tag) __attribute__((always_inline)) {
         constexpr int KGV = decltype(group_tag)::value;
         issue_a();
 #pragma unroll
         for (int s = 0; s < kStages; ++s) issue_b(s);
-        AChunk a_cur[FM];
-        half16_t bv_even[FN], bv_odd[FN];
-        half8_t av_even[FM], av_odd[FM];
+        AChunk a_cur[FM], a_next[FM];
+        u32x8_t bv_even[FN], bv_odd[FN];
+        u32x4_t av_even[FM], av_odd[FM];
         wait_vmcnt<3 * NL>();  // A(0) and B(0) have landed
         __builtin_amdgcn_s_barrier();
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) a_cur[fm] = load_a_chunk_lds(a_frag_lds[fm], lane);
-        read_frags(0, KGV, bv_even);
-        expand_frags<KGV>(a_cur, one, av_even);
+#pragma unroll
+        for (int r = 0; r < PIECES; ++r) read_piece(0, KGV, r, bv_even);
+#pragma unroll
+        for (int g = 0; g < 4 * FM; ++g) av_even[g / 4][g % 4] = expand_sign_register<KGV>(a_cur[g / 4], one, g % 4);
 #define ONEBIT_GROUP_STAGE(S, WAITCNT, ISSUE_A, BV, AV, BV_NEXT, AV_NEXT)                                         \
         {                                                                                                        \
           wait_vmcnt_lgkm0<(WAITCNT)>();                                                                         \
           __builtin_amdgcn_s_barrier();                                                                          \
-          if (ISSUE_A) issue_a();                                                                                \
-          issue_b(S);                                                                                            \
-          read_frags(((S) + 1) % kStages, KGV, BV_NEXT);                                                         \
-          if constexpr ((S) < kStages - 1) {                                                                     \
-            expand_frags_here<2 * ((S) + 1) + KGV>(a_cur, one, AV_NEXT);                                              \
-            mfma_frags<2 * (S) + KGV>(a_cur, AV, BV, acc);                                                       \
-          } else {                                                                                               \
-            AChunk a_next[FM];                                                                                   \
+          if constexpr ((S) == kStages - 1) {                                                                    \
             _Pragma("unroll") for (int fm = 0; fm < FM; ++fm) a_next[fm] = load_a_chunk_lds(a_frag_lds[fm], lane); \
-            expand_frags_here<KGV>(a_next, one, AV_NEXT);                                                           \
-            mfma_frags<2 * (S) + KGV>(a_cur, AV, BV, acc);                                                       \
+            __builtin_amdgcn_sched_barrier(0);                                                                   \
+          }                                                                                                      \
+          mfma_frags_fused<2 * (S) + KGV, false>(a_cur, AV, BV, acc, [&](int slot) __attribute__((always_inline)) { \
+            ONEBIT_COPY_SLOT(S, ISSUE_A)                                                                         \
+            if constexpr ((S) < kStages - 1) {                                                                   \
+              ONEBIT_FETCH_SLOT((S) + 1, KGV, BV_NEXT, 2 * ((S) + 1) + KGV, a_cur, AV_NEXT)                      \
+            } else {                                                                                             \
+              ONEBIT_FETCH_SLOT(0, KGV, BV_NEXT, KGV, a_next, AV_NEXT)                                           \
+            }                                                                                                    \
+          });                                                                                                    \
+          if constexpr ((S) == kStages - 1) {                                                                    \
             _Pragma("unroll") for (int fm = 0; fm < FM; ++fm) a_cur[fm] = a_next[fm];                            \
           }                                                                                                      \
-          __builtin_amdgcn_sched_barrier(0);                                                                     \
         }
-        for (int kc = chunk_begin; kc < chunk_end; ++kc) {
+        auto chunk_body = [&](auto full_tag) __attribute__((always_inline)) {
+          constexpr bool FULL = decltype(full_tag)::value;
           ONEBIT_GROUP_STAGE(0, 2 * NL, true, bv_even, av_even, bv_odd, av_odd)
           ONEBIT_GROUP_STAGE(1, 2 * NL + NA, false, bv_odd, av_odd, bv_even, av_even)
           ONEBIT_GROUP_STAGE(2, 2 * NL + NA, false, bv_even, av_even, bv_odd, av_odd)
           ONEBIT_GROUP_STAGE(3, 2 * NL, false, bv_odd, av_odd, bv_even, av_even)
-        }
+        };
+        int kc = chunk_begin;
+        for (; kc < full_end; ++kc) chunk_body(std::true_type{});
+        for (; kc < chunk_end; ++kc) chunk_body(std::false_type{});
 #undef ONEBIT_GROUP_STAGE
         wait_vmcnt<0>();  // drain the copies issued past the end before the LDS is released
       };
       if (kg == 0) run(std::integral_constant<int, 0>{});
       else run(std::integral_constant<int, 1>{});
+#undef ONEBIT_FETCH_SLOT
+#undef ONEBIT_COPY_SLOT
       smfmac_drain();
       __syncthreads();  // the stage ring is free
       if constexpr (kSplitEpilogue) {
