@@ -850,6 +850,53 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
       // The pieces of C that a lane will need for one 32-row block are requested together, before the block's sums
       // travel through the scratch, so that one memory latency per block is paid instead of one per piece.
       const bool use_c = p.beta != 0.f;
+      if (p.d_f16 && !use_c && WCOLS >= 8) {
+        // fp16 result without C: alpha * sum is rounded in the accumulator layout, where registers v and v + 1 (v even)
+        // of a lane are rows r and r + 1 of one column; the two halves go through the scratch as one word (a quarter of
+        // the LDS traffic of the fp32 form). A lane then reads eight such words (columns c .. c + 7 of a row pair),
+        // separates low and high halves and stores 16 bytes of row r and 16 bytes of row r + 1.
+        uint32_t* const words = reinterpret_cast<uint32_t*>(scratch);  // [16 row pairs][WCOLS]
+        constexpr int PER_PAIR = WCOLS / 8;            // 8-column pieces per row pair
+        constexpr int TASKS = 16 * PER_PAIR;           // (row pair, piece) per 32-row block
+        constexpr int ITERS = (TASKS + 63) / 64;
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm) {
+          if (!finishes(fm)) continue;  // the other K group stores this fragment
+          const int row_base = row0 + fm * 32;
+#pragma unroll
+          for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+              const _Float16 h0 = (_Float16)(p.alpha * acc[fm][fn][2 * q]);
+              const _Float16 h1 = (_Float16)(p.alpha * acc[fm][fn][2 * q + 1]);
+              const uint32_t w = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
+              // rows 8 (q / 2) + 4 (lane / 32) + 2 (q % 2) and the next: row pair 4 (q / 2) + 2 (lane / 32) + q % 2
+              words[(4 * (q / 2) + (row_lane >> 1) + (q & 1)) * WCOLS + fn * 32 + col_lane] = w;
+            }
+#pragma unroll
+          for (int it = 0; it < ITERS; ++it) {
+            const int task = it * 64 + lane;
+            if (TASKS % 64 != 0 && task >= TASKS) break;
+            const int pair = task / PER_PAIR, c8 = (task % PER_PAIR) * 8;
+            const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(words + pair * WCOLS + c8);
+            const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(words + pair * WCOLS + c8 + 4);
+            const uint32_t d[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            u32x4_t even_row, odd_row;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              even_row[j] = __builtin_amdgcn_perm(d[2 * j + 1], d[2 * j], 0x05040100u);  // low halves
+              odd_row[j] = __builtin_amdgcn_perm(d[2 * j + 1], d[2 * j], 0x07060302u);   // high halves
+            }
+            const int row = row_base + 2 * pair, col = col0 + c8;
+            if (col < p.n) {
+              _Float16* const out = reinterpret_cast<_Float16*>(d_out) + (size_t)row * p.n + col;
+              if (row < row_limit) *reinterpret_cast<u32x4_t*>(out) = even_row;
+              if (row + 1 < row_limit) *reinterpret_cast<u32x4_t*>(out + p.n) = odd_row;
+            }
+          }
+        }
+        return;
+      }
 #pragma unroll
       for (int fm = 0; fm < FM; ++fm) {
         if (!finishes(fm)) continue;  // the other K group stores this fragment
