@@ -311,8 +311,10 @@ __device__ __forceinline__ void mfma_frags_fused(const AChunk (&a)[FM], const u3
   for (int fm = 0; fm < FM; ++fm)
 #pragma unroll
     for (int fn = 0; fn < FN; ++fn) {
+      __builtin_amdgcn_s_setprio(1);  // the wavefront that is about to issue an SMFMAC wins the arbitration on its SIMD
       acc[fm][fn] = smfmac_step<STEP, PINNED>(a[fm], __builtin_bit_cast(half8_t, av[fm]),
                                               __builtin_bit_cast(half16_t, bv[fn]), acc[fm][fn]);
+      __builtin_amdgcn_s_setprio(0);
       __builtin_amdgcn_sched_barrier(0);
       fetch(fm * FN + fn);
       __builtin_amdgcn_sched_barrier(0);
