@@ -849,6 +849,16 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
       constexpr int WCOLS = FN * 32;                   // columns of the wavefront's tile
       float* scratch = reinterpret_cast<float*>(smem) + wave * (32 * WCOLS);
       const int col_lane = lane & 31, row_lane = 4 * (lane >> 5);
+      // Column swizzle of the scratch against bank conflicts, the same for rows of floats and for row pairs of packed
+      // halves: line L keeps its 16-byte slots swapped in pairs when L is odd (two consecutive lines are read by one
+      // group of sixteen lanes: they then touch different banks), and, with lines of 256 bytes or more, its two halves of
+      // 128 bytes swapped when bit 2 (rows) or bit 1 (row pairs) of L is set (the upper half-wavefront writes the line
+      // that many below the lower half's).
+      constexpr int kHalfSwap = WCOLS >= 64 ? 32 : 0;
+      const int half_write = (lane >> 5) * kHalfSwap;  // the writer's own half swap; (line & 1) << 2 is per register
+      auto read_swizzle = [&](int line, int half_bit) __attribute__((always_inline)) {
+        return ((line & 1) << 2) ^ (((line >> half_bit) & 1) * kHalfSwap);
+      };
       // The pieces of C that a lane will need for one 32-row block are requested together, before the block's sums
       // travel through the scratch, so that one memory latency per block is paid instead of one per piece.
       const bool use_c = p.beta != 0.f;
@@ -873,15 +883,16 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
               const _Float16 h1 = (_Float16)(p.alpha * acc[fm][fn][2 * q + 1]);
               const uint32_t w = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
               // rows 8 (q / 2) + 4 (lane / 32) + 2 (q % 2) and the next: row pair 4 (q / 2) + 2 (lane / 32) + q % 2
-              words[(4 * (q / 2) + (row_lane >> 1) + (q & 1)) * WCOLS + fn * 32 + col_lane] = w;
+              words[(4 * (q / 2) + (row_lane >> 1) + (q & 1)) * WCOLS + ((fn * 32 + col_lane) ^ half_write ^ ((q & 1) << 2))] = w;
             }
 #pragma unroll
           for (int it = 0; it < ITERS; ++it) {
             const int task = it * 64 + lane;
             if (TASKS % 64 != 0 && task >= TASKS) break;
             const int pair = task / PER_PAIR, c8 = (task % PER_PAIR) * 8;
-            const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(words + pair * WCOLS + c8);
-            const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(words + pair * WCOLS + c8 + 4);
+            const int sw = read_swizzle(pair, 1);
+            const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(words + pair * WCOLS + (c8 ^ sw));
+            const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(words + pair * WCOLS + ((c8 + 4) ^ sw));
             const uint32_t d[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
             u32x4_t even_row, odd_row;
 #pragma unroll
@@ -928,14 +939,15 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
           for (int fn = 0; fn < FN; ++fn)
 #pragma unroll
             for (int v = 0; v < 16; ++v)
-              scratch[(8 * (v / 4) + row_lane + (v % 4)) * WCOLS + fn * 32 + col_lane] = acc[fm][fn][v];
+              scratch[(8 * (v / 4) + row_lane + (v % 4)) * WCOLS + ((fn * 32 + col_lane) ^ half_write ^ ((v & 1) << 2))] = acc[fm][fn][v];
 #pragma unroll
           for (int it = 0; it < ITERS; ++it) {
             const int piece = it * 64 + lane;
             const int r = piece / PER_ROW, c8 = (piece % PER_ROW) * 8;
             const int row = row_base + r, col = col0 + c8;
-            const float4 lo = *reinterpret_cast<const float4*>(scratch + r * WCOLS + c8);
-            const float4 hi = *reinterpret_cast<const float4*>(scratch + r * WCOLS + c8 + 4);
+            const int sw = read_swizzle(r, 2);
+            const float4 lo = *reinterpret_cast<const float4*>(scratch + r * WCOLS + (c8 ^ sw));
+            const float4 hi = *reinterpret_cast<const float4*>(scratch + r * WCOLS + ((c8 + 4) ^ sw));
             float x[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
             if (row < row_limit && col < p.n) {
               const size_t o = (size_t)row * p.n + col;
@@ -982,13 +994,13 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
           for (int fn = 0; fn < FN; ++fn)
 #pragma unroll
             for (int v = 0; v < 16; ++v)
-              scratch[(8 * (v / 4) + row_lane + (v % 4)) * WCOLS + fn * 32 + col_lane] = acc[fm][fn][v];
+              scratch[(8 * (v / 4) + row_lane + (v % 4)) * WCOLS + ((fn * 32 + col_lane) ^ half_write ^ ((v & 1) << 2))] = acc[fm][fn][v];
 #pragma unroll
           for (int it = 0; it < ITERS; ++it) {
             const int piece = it * 64 + lane;
             const int r = piece / PER_ROW, c4 = (piece % PER_ROW) * 4;
             const int row = row_base + r, col = col0 + c4;
-            const float4 a4 = *reinterpret_cast<const float4*>(scratch + r * WCOLS + c4);
+            const float4 a4 = *reinterpret_cast<const float4*>(scratch + r * WCOLS + (c4 ^ read_swizzle(r, 2)));
             float x[4] = {a4.x, a4.y, a4.z, a4.w};
             if (row < row_limit && col < p.n) {
               const size_t o = (size_t)row * p.n + col;
