@@ -868,9 +868,14 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
         // the LDS traffic of the fp32 form). A lane then reads eight such words (columns c .. c + 7 of a row pair),
         // separates low and high halves and stores 16 bytes of row r and 16 bytes of row r + 1.
         uint32_t* const words = reinterpret_cast<uint32_t*>(scratch);  // [16 row pairs][WCOLS]
+        typedef float float2v __attribute__((ext_vector_type(2)));
+        typedef _Float16 half2v __attribute__((ext_vector_type(2)));
         constexpr int PER_PAIR = WCOLS / 8;            // 8-column pieces per row pair
         constexpr int TASKS = 16 * PER_PAIR;           // (row pair, piece) per 32-row block
         constexpr int ITERS = (TASKS + 63) / 64;
+        // alpha == 1 is tested once per wavefront, not per value: two copies of the loop
+        auto packed_turn = [&](auto scale_tag) __attribute__((always_inline)) {
+        constexpr bool SCALE = decltype(scale_tag)::value;
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) {
           if (!finishes(fm)) continue;  // the other K group stores this fragment
@@ -879,9 +884,9 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
           for (int fn = 0; fn < FN; ++fn)
 #pragma unroll
             for (int q = 0; q < 8; ++q) {
-              const _Float16 h0 = (_Float16)(p.alpha * acc[fm][fn][2 * q]);
-              const _Float16 h1 = (_Float16)(p.alpha * acc[fm][fn][2 * q + 1]);
-              const uint32_t w = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
+              float2v x = {acc[fm][fn][2 * q], acc[fm][fn][2 * q + 1]};  // one packed conversion per register pair
+              if constexpr (SCALE) x = float2v{p.alpha * x.x, p.alpha * x.y};
+              const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, half2v));
               // rows 8 (q / 2) + 4 (lane / 32) + 2 (q % 2) and the next: row pair 4 (q / 2) + 2 (lane / 32) + q % 2
               words[(4 * (q / 2) + (row_lane >> 1) + (q & 1)) * WCOLS + ((fn * 32 + col_lane) ^ half_write ^ ((q & 1) << 2))] = w;
             }
@@ -908,6 +913,9 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
             }
           }
         }
+        };
+        if (p.alpha != 1.f) packed_turn(std::true_type{});
+        else packed_turn(std::false_type{});
         return;
       }
 #pragma unroll
