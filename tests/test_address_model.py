@@ -430,3 +430,97 @@ def test_the_model_catches_an_out_of_range_access():
             check_gemm(1024, 512, 1024, 9, 1, False)
     finally:
         globals()["prepared_bytes"] = real
+
+
+# ---- the epilogue's turn through the LDS scratch (gemm_kernel, coalesced form) ------------------------------------
+# Restates the index arithmetic of the two forms: fp32 rows [32][WCOLS] and packed fp16 row pairs [16][WCOLS], both with
+# the column swizzle (16-byte slots swapped in pairs on odd lines, 128-byte halves swapped when bit 2 of the row / bit 1
+# of the row pair is set and a line has at least 64 columns).
+
+def _half_swap(wcols):
+    return 32 if wcols >= 64 else 0
+
+
+def _scratch_rows_model(fn_count):
+    """(writes, reads) of the fp32 form for one 32-row block: dicts word -> (row, column) written / read."""
+    wcols = fn_count * 32
+    writes, reads = {}, {}
+    for lane in range(64):
+        col_lane, row_lane = lane & 31, 4 * (lane >> 5)
+        half_write = (lane >> 5) * _half_swap(wcols)
+        for fn in range(fn_count):
+            for v in range(16):
+                row = 8 * (v // 4) + row_lane + v % 4
+                word = row * wcols + ((fn * 32 + col_lane) ^ half_write ^ ((v & 1) << 2))
+                assert word not in writes
+                writes[word] = (row, fn * 32 + col_lane)
+    per_row = wcols // 8
+    for it in range(32 * per_row // 64):
+        for lane in range(64):
+            piece = it * 64 + lane
+            r, c8 = piece // per_row, (piece % per_row) * 8
+            sw = ((r & 1) << 2) ^ (((r >> 2) & 1) * _half_swap(wcols))
+            for part, base in ((0, c8), (1, c8 + 4)):
+                for j in range(4):
+                    reads[r * wcols + (base ^ sw) + j] = (r, base + j)
+    return wcols, writes, reads
+
+
+def _scratch_pairs_model(fn_count):
+    """the packed form: word -> (row pair, column)."""
+    wcols = fn_count * 32
+    writes, reads = {}, {}
+    for lane in range(64):
+        col_lane, row_lane = lane & 31, 4 * (lane >> 5)
+        half_write = (lane >> 5) * _half_swap(wcols)
+        for fn in range(fn_count):
+            for q in range(8):
+                pair = 4 * (q // 2) + (row_lane >> 1) + (q & 1)
+                rows = 8 * (q // 2) + row_lane + 2 * (q % 2)   # registers 2q, 2q + 1 of the accumulator layout
+                assert rows == 2 * pair
+                word = pair * wcols + ((fn * 32 + col_lane) ^ half_write ^ ((q & 1) << 2))
+                assert word not in writes
+                writes[word] = (pair, fn * 32 + col_lane)
+    per_pair = wcols // 8
+    tasks = 16 * per_pair
+    for it in range((tasks + 63) // 64):
+        for lane in range(64):
+            task = it * 64 + lane
+            if task >= tasks:
+                continue
+            pair, c8 = task // per_pair, (task % per_pair) * 8
+            sw = ((pair & 1) << 2) ^ (((pair >> 1) & 1) * _half_swap(wcols))
+            for base in (c8, c8 + 4):
+                for j in range(4):
+                    reads[pair * wcols + (base ^ sw) + j] = (pair, base + j)
+    return wcols, writes, reads
+
+
+@pytest.mark.parametrize("fn_count", [1, 2, 4])
+@pytest.mark.parametrize("model,lines", [(_scratch_rows_model, 32), (_scratch_pairs_model, 16)])
+def test_epilogue_scratch_is_written_once_and_read_back_where_it_was_written(model, lines, fn_count):
+    wcols, writes, reads = model(fn_count)
+    assert sorted(writes) == list(range(lines * wcols))          # every word of the wavefront's scratch, once, in range
+    assert reads == writes                                       # a reader finds (line, column) where the writer put it
+
+
+def test_epilogue_scratch_swizzle_avoids_bank_conflicts():
+    # The tiles the planner uses have 64-column wavefront tiles. 64 banks of 4 bytes. A 4-byte store instruction: the 32
+    # lanes of each half-wavefront touch 32 different banks and the two halves touch different ones. A 16-byte read: the
+    # 16 lanes served together (two lines) touch 64 different banks.
+    wcols = 64
+    for v in range(16):
+        banks = []
+        for lane in range(64):
+            row = 8 * (v // 4) + 4 * (lane >> 5) + v % 4
+            word = row * wcols + ((lane & 31) ^ ((lane >> 5) * 32) ^ ((v & 1) << 2))
+            banks.append(word % 64)
+        assert len(set(banks)) == 64
+    per_row = wcols // 8
+    for group in range(4):
+        banks = []
+        for lane in range(16 * group, 16 * group + 16):
+            r, c8 = lane // per_row, (lane % per_row) * 8
+            sw = ((r & 1) << 2) ^ (((r >> 2) & 1) * 32)
+            banks += [(r * wcols + (c8 ^ sw) + j) % 64 for j in range(4)]
+        assert len(set(banks)) == 64
