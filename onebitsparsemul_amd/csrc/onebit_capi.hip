@@ -228,6 +228,14 @@ GemmPlan plan_gemm(int m, int n, int k, int compute_units) {
       consider(t, s);
     }
   }
+  // With every compute unit busy the 512 x 128 tile is bound by power, and the same tile built on the 16x16x64 SMFMAC
+  // (four wavefronts, one per SIMD) draws less of it per product: 3-5 % faster from about one full round of tiles on
+  // (8192^3, 4096^3, 25600^3; 28672 x 512 x 8192 with 224 tiles: 102.9 against 107.0 us), slower when part of the chip
+  // idles and the schedule decides (4096 x 3072 x 4096 with 192 tiles: 51.2 against 50.6; 11008 x 768 x 4096: 49 against 41).
+  if (best.tile == onebit::kTile512x128w8 && best.splits == 1) {
+    const long tiles = (long)((m + 511) / 512) * ((n + 127) / 128);
+    if (tiles * 20 >= 17L * compute_units) best.tile = onebit::kTile512x128m16;  // from 85 % of a round on
+  }
   return best;
 }
 
@@ -516,7 +524,7 @@ int onebit_sparse_linear_prepared(const void* prepared, const void* x, const voi
   if (!prepared || !x || !y) return fail(ONEBIT_ERR_ARGUMENT, "null operand pointer");
   if ((reinterpret_cast<uintptr_t>(x) & 15) != 0) return fail(ONEBIT_ERR_ARGUMENT, "x must be 16-byte aligned");
   const int kc_total = (k + onebit::kChunkK - 1) / onebit::kChunkK;
-  const LaunchPlan plan = choose_launch(m, tokens, k, true, current_compute_units());
+  LaunchPlan plan = choose_launch(m, tokens, k, true, current_compute_units());
   if ((size_t)k * 256 * 2 >= (size_t(1) << 32))
     return fail(ONEBIT_ERR_ARGUMENT, "the token-major form addresses x with 32-bit offsets inside a tile of 256 tokens: "
                                      "k = %d is beyond its limit of 8388607", k);
@@ -535,6 +543,8 @@ int onebit_sparse_linear_prepared(const void* prepared, const void* x, const voi
     ONEBIT_HIP(onebit::launch_skinny_tokens(args, plan.rows_or_tile, static_cast<hipStream_t>(stream)));
     return ONEBIT_OK;
   }
+  // the linear layer's form has no 16x16x64 variant: the same tile on eight wavefronts
+  if (plan.rows_or_tile == onebit::kTile512x128m16) plan.rows_or_tile = onebit::kTile512x128w8;
   switch (plan.rows_or_tile) {
     case onebit::kTile256x128w: case onebit::kTile128x128s: case onebit::kTile512x128w8: case onebit::kTile256x128w8:
     case onebit::kTile128x128w8: case onebit::kTile64x128: case onebit::kTile128x128k2: case onebit::kTile64x128k2: break;

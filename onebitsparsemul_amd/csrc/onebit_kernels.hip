@@ -326,8 +326,9 @@ __device__ __attribute__((aligned(16))) uint32_t g_zero16[4] = {0, 0, 0, 0};
 
 // TOKENS (with DMA only): the linear-layer form. p.b is x (p.n tokens x p.k, token-major), p.d is y (p.n tokens x
 // p.m), the epilogue is y = acc + bias; a tile column is a token.
-template <int WM, int WN, int FM, int FN, bool DMA, bool TOKENS = false, int KG = 1>
+template <int WM, int WN, int FM, int FN, bool DMA, bool TOKENS = false, int KG = 1, bool M16 = false>
 __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmArgs p) {
+  static_assert(!M16 || (DMA && !TOKENS && KG == 1 && WN == 1 && FM == 4 && FN == 4), "the 16x16x64 form exists for the 512x128 four-wavefront tile");
   static_assert(DMA || !TOKENS, "the token-major form uses the asynchronous copies");
   static_assert(DMA || KG == 1, "the two-group form uses the asynchronous copies");
   using TS = TileShape<WM, WN, FM, FN, KG>;
@@ -378,13 +379,19 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
   const char* const wave_image = smem + wn * FN * (32 * kStageK * 2);  // first token row of this wavefront in stage 0
 
   const uint32_t one = packed_one_in_vgpr();
-  float16_t acc[FM][FN];
+  // 32x32x32 form: FM x FN tiles of 32 x 32; 16x16x64 form: 2 FM x 2 FN tiles of 16 x 16 (the other array has one element)
+  float16_t acc[M16 ? 1 : FM][M16 ? 1 : FN];
+  float4v_t acc16[M16 ? 2 * FM : 1][M16 ? 2 * FN : 1];
 #pragma unroll
-  for (int fm = 0; fm < FM; ++fm)
+  for (int fm = 0; fm < (M16 ? 1 : FM); ++fm)
 #pragma unroll
-    for (int fn = 0; fn < FN; ++fn)
+    for (int fn = 0; fn < (M16 ? 1 : FN); ++fn)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[fm][fn][v] = 0.f;
+#pragma unroll
+  for (int rt = 0; rt < (M16 ? 2 * FM : 1); ++rt)
+#pragma unroll
+    for (int ct = 0; ct < (M16 ? 2 * FN : 1); ++ct) acc16[rt][ct] = float4v_t{0.f, 0.f, 0.f, 0.f};
 
   const int stages_total = (p.k + kStageK - 1) / kStageK;
   const int chunks = (stages_total + kStages - 1) / kStages;
@@ -542,7 +549,144 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
     // chunk kc copies the stages of chunk kc + 1: they are whole while (kc + 2) * 256 <= K
     const int full_end = p.k / kChunkK - 1 < chunk_end ? p.k / kChunkK - 1 : chunk_end;
 
-    if constexpr (KG == 1) {
+    if constexpr (M16) {
+      // ---- 16x16x64 form of the K loop (one wavefront per SIMD, wave tile 128 x 128 = 8 x 8 tiles of 16 x 16) ----
+      // One SMFMAC covers a whole 64-row stage. A-operand lane (row l % 16, group l / 16) holds the kept values of K
+      // positions [16 g, 16 g + 16) of the stage, i.e. what lane row + 32 (g % 2) of the prepared block holds for K step
+      // 2 S + g / 2; B-operand lane (column l % 16, group g) holds K rows 8 g ... 8 g + 7 of both 32-row halves.
+      // First half of a stage (before the barrier): row tiles 0-3 against all column tiles, the signs of the next row
+      // tile and of row tiles 4-7 expanded between the SMFMACs. Second half: column tile by column tile against row
+      // tiles 4-7; a column tile's fragment registers are free after its four SMFMACs and take the next stage's
+      // fragment, which the barrier has just published.
+      constexpr int RT = 2 * FM, CT = 2 * FN;
+      const int g16 = lane >> 4, c16 = lane & 15;
+      const int brow = 8 * g16 + (c16 >> 2);  // + 0, 4, 32, 36
+      const int brow_off = brow * (BN * 2);
+      int ct_off[CT];
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        ct_off[ct] = (((2 * (wn * CT + ct) + ((c16 & 3) >> 1)) ^ chunk_swizzle<BN>(brow)) << 4) + (c16 & 1) * 8;
+      auto read_b16 = [&](int ring_slot, int ct, int q, u32x8_t* bv) __attribute__((always_inline)) {
+        const int row_const = 4 * (q & 1) + 32 * (q >> 1);
+        const u32x2_t t = lds_read_tr16(smem + ring_slot * TS::STAGE_BYTES + brow_off + row_const * (BN * 2) + ct_off[ct]);
+        bv[ct][2 * q] = t.x;
+        bv[ct][2 * q + 1] = t.y;
+      };
+      // per row tile: metadata of stages 0,1 and 2,3 (16 bits each, chosen by ABID), sign words of stages 0,1 and 2,3
+      struct ATile { uint32_t idx01, idx23, w01, w23; };
+      const uint32_t half_select = (g16 >> 1) ? 0x07060302u : 0x05040100u;
+      const int sign_shift = 4 * (g16 >> 1);
+      auto gather_a = [&](int rt) __attribute__((always_inline)) {
+        const char* block = a_frag_lds[rt >> 1];
+        const int holder = c16 + 16 * (rt & 1) + 32 * (g16 & 1);
+        const u32x4_t meta = *reinterpret_cast<const u32x4_t*>(block + holder * 16);
+        const u32x2_t sign = *reinterpret_cast<const u32x2_t*>(block + kSignOffset + holder * 8);
+        ATile t;
+        t.idx01 = __builtin_amdgcn_perm(meta.y, meta.x, half_select);
+        t.idx23 = __builtin_amdgcn_perm(meta.w, meta.z, half_select);
+        t.w01 = sign.x << sign_shift;
+        t.w23 = sign.y << sign_shift;
+        return t;
+      };
+      // register p (kept values 2p, 2p+1) of the expanded signs of stage S
+      auto expand16 = [&](const ATile& t, int S, int p_) __attribute__((always_inline)) {
+        const uint32_t w = S < 2 ? t.w01 : t.w23;
+        uint32_t v = ((w << (8 * (S & 1) + p_)) & 0x80008000u) | one;
+        asm volatile("" : "+v"(v));
+        return v;
+      };
+      auto mma16 = [&](float4v_t& c, const u32x4_t& av, const u32x8_t& bv, const ATile& t, int S) __attribute__((always_inline)) {
+        const uint32_t idx = S < 2 ? t.idx01 : t.idx23;
+        const half8_t a8 = __builtin_bit_cast(half8_t, av);
+        const half16_t b16 = __builtin_bit_cast(half16_t, bv);
+        // accumulators tied to accumulation registers, as in smfmac_step
+        if ((S & 1) == 0) asm("v_smfmac_f32_16x16x64_f16 %0, %1, %2, %3" : "+a"(c) : "v"(a8), "v"(b16), "v"(idx));
+        else asm("v_smfmac_f32_16x16x64_f16 %0, %1, %2, %3 abid:1" : "+a"(c) : "v"(a8), "v"(b16), "v"(idx));
+      };
+
+      issue_a();
+#pragma unroll
+      for (int s = 0; s < kStages; ++s) issue_b(s);
+      ATile a_cur[RT];
+      u32x8_t bv[CT];
+      u32x4_t av_roll[2], av_hi[RT / 2];
+      wait_vmcnt<3 * NL>();  // A(0) and B(0) have landed
+      __builtin_amdgcn_s_barrier();
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) a_cur[rt] = gather_a(rt);
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) read_b16(0, ct, q, bv);
+#pragma unroll
+      for (int p_ = 0; p_ < 4; ++p_) av_roll[0][p_] = expand16(a_cur[0], 0, p_);
+
+      auto chunk_body = [&](auto full_tag) __attribute__((always_inline)) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        constexpr int SLOTS = RT / 2 * CT;  // SMFMACs per half stage (shadows the 32x32x32 form's count for the copy macro)
+        auto stage = [&](auto s_tag, auto wait_tag, auto issue_a_tag) __attribute__((always_inline)) {
+          constexpr int S = decltype(s_tag)::value;
+          constexpr int WAITCNT = decltype(wait_tag)::value;
+          constexpr bool ISSUE_A = decltype(issue_a_tag)::value;
+          // first half: row tiles 0-3
+#pragma unroll
+          for (int rt = 0; rt < RT / 2; ++rt)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+              mma16(acc16[rt][ct], av_roll[rt & 1], bv[ct], a_cur[rt], S);
+              __builtin_amdgcn_sched_barrier(0);
+              // this slot's share of the eight registers to expand: the next row tile's four, then row tile 4 + rt's four
+#pragma unroll
+              for (int e = ct * 8 / CT; e < (ct + 1) * 8 / CT; ++e) {
+                if (e < 4) {
+                  if (rt + 1 < RT / 2) av_roll[(rt + 1) & 1][e] = expand16(a_cur[rt + 1], S, e);
+                } else {
+                  av_hi[rt][e - 4] = expand16(a_cur[RT / 2 + rt], S, e - 4);
+                }
+              }
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          wait_vmcnt_lgkm0<WAITCNT>();  // copies of stage S+1 landed
+          __builtin_amdgcn_s_barrier();
+          if constexpr (S == kStages - 1) {
+            // the next chunk of A is readable after this stage's barrier; row tiles 0-3 are done with this chunk
+#pragma unroll
+            for (int rt = 0; rt < RT / 2; ++rt) a_cur[rt] = gather_a(rt);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          // second half: column tile by column tile against row tiles 4-7
+#pragma unroll
+          for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int rl = 0; rl < RT / 2; ++rl) {
+              const int slot = ct * (RT / 2) + rl;
+              mma16(acc16[RT / 2 + rl][ct], av_hi[rl], bv[ct], a_cur[RT / 2 + rl], S);
+              __builtin_amdgcn_sched_barrier(0);
+              ONEBIT_COPY_SLOT(S, ISSUE_A)
+              // the fragment of column tile ct - 1 for the next stage, one read behind each of this tile's SMFMACs
+              if (ct >= 1) read_b16((S + 1) % kStages, ct - 1, rl, bv);
+              // signs of row tile 0 of the next stage
+              if (ct == CT - 1) av_roll[0][rl] = expand16(a_cur[0], (S + 1) % kStages, rl);
+              __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+          for (int q = 0; q < 4; ++q) read_b16((S + 1) % kStages, CT - 1, q, bv);
+          if constexpr (S == kStages - 1) {
+#pragma unroll
+            for (int rt = RT / 2; rt < RT; ++rt) a_cur[rt] = gather_a(rt);  // row tiles 4-7 are done with this chunk
+          }
+        };
+        using std::integral_constant;
+        stage(integral_constant<int, 0>{}, integral_constant<int, 2 * NL>{}, std::true_type{});        // waits for B(4c+1)
+        stage(integral_constant<int, 1>{}, integral_constant<int, 2 * NL + NA>{}, std::false_type{});  // B(4c+2)
+        stage(integral_constant<int, 2>{}, integral_constant<int, 2 * NL + NA>{}, std::false_type{});  // B(4c+3)
+        stage(integral_constant<int, 3>{}, integral_constant<int, 2 * NL>{}, std::false_type{});       // B(4c+4)
+      };
+      int kc = chunk_begin;
+      for (; kc < full_end; ++kc) chunk_body(std::true_type{});
+      for (; kc < chunk_end; ++kc) chunk_body(std::false_type{});
+      wait_vmcnt<0>();  // drain the copies issued past the end before the LDS is released
+    } else if constexpr (KG == 1) {
       // The barrier sits in the middle of each stage s: it publishes stage s+1 (read right after it) and frees the ring
       // slot of stage s (all of its reads were issued in the first half).
       issue_a();
@@ -855,7 +999,31 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
       // 128 bytes swapped when bit 2 (rows) or bit 1 (row pairs) of L is set (the upper half-wavefront writes the line
       // that many below the lower half's).
       constexpr int kHalfSwap = WCOLS >= 64 ? 32 : 0;
-      const int half_write = (lane >> 5) * kHalfSwap;  // the writer's own half swap; (line & 1) << 2 is per register
+      // The accumulators of 32-row block fm into the scratch. 32x32x32 form: register v of fragment fn is row
+      // 8 (v / 4) + 4 (lane / 32) + v % 4, column 32 fn + lane % 32; 16x16x64 form: register v of tile (2 fm + rh, ct) is
+      // row 16 rh + 4 (lane / 16) + v, column 16 ct + lane % 16. In both, bit 2 of the row is one bit of the lane
+      // (the writer's own half swap) and bit 0 of the row is bit 0 of v.
+      const int g16 = lane >> 4, c16 = lane & 15;
+      const int half_write = (M16 ? (g16 & 1) : (lane >> 5)) * kHalfSwap;
+      auto store_rows = [&](int fm) __attribute__((always_inline)) {
+        if constexpr (M16) {
+#pragma unroll
+          for (int rh = 0; rh < 2; ++rh)
+#pragma unroll
+            for (int ct = 0; ct < 2 * FN; ++ct)
+#pragma unroll
+              for (int v = 0; v < 4; ++v)
+                scratch[(16 * rh + 4 * g16 + v) * WCOLS + ((ct * 16 + c16) ^ half_write ^ ((v & 1) << 2))] =
+                    acc16[2 * fm + rh][ct][v];
+        } else {
+#pragma unroll
+          for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+              scratch[(8 * (v / 4) + row_lane + (v % 4)) * WCOLS + ((fn * 32 + col_lane) ^ half_write ^ ((v & 1) << 2))] =
+                  acc[fm][fn][v];
+        }
+      };
       auto read_swizzle = [&](int line, int half_bit) __attribute__((always_inline)) {
         return ((line & 1) << 2) ^ (((line >> half_bit) & 1) * kHalfSwap);
       };
@@ -880,16 +1048,31 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
         for (int fm = 0; fm < FM; ++fm) {
           if (!finishes(fm)) continue;  // the other K group stores this fragment
           const int row_base = row0 + fm * 32;
+          auto pack = [&](float x0, float x1) __attribute__((always_inline)) {  // one packed conversion per register pair
+            float2v x = {x0, x1};
+            if constexpr (SCALE) x = float2v{p.alpha * x.x, p.alpha * x.y};
+            return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, half2v));
+          };
+          if constexpr (M16) {
+            // registers (0, 1) and (2, 3) of a tile: rows 16 rh + 4 (lane / 16) + 2 h and the next, row pair
+            // 8 rh + 2 (lane / 16) + h
 #pragma unroll
-          for (int fn = 0; fn < FN; ++fn)
+            for (int rh = 0; rh < 2; ++rh)
 #pragma unroll
-            for (int q = 0; q < 8; ++q) {
-              float2v x = {acc[fm][fn][2 * q], acc[fm][fn][2 * q + 1]};  // one packed conversion per register pair
-              if constexpr (SCALE) x = float2v{p.alpha * x.x, p.alpha * x.y};
-              const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, half2v));
-              // rows 8 (q / 2) + 4 (lane / 32) + 2 (q % 2) and the next: row pair 4 (q / 2) + 2 (lane / 32) + q % 2
-              words[(4 * (q / 2) + (row_lane >> 1) + (q & 1)) * WCOLS + ((fn * 32 + col_lane) ^ half_write ^ ((q & 1) << 2))] = w;
-            }
+              for (int ct = 0; ct < 2 * FN; ++ct)
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+                  words[(8 * rh + 2 * g16 + h) * WCOLS + ((ct * 16 + c16) ^ half_write ^ (h << 2))] =
+                      pack(acc16[2 * fm + rh][ct][2 * h], acc16[2 * fm + rh][ct][2 * h + 1]);
+          } else {
+#pragma unroll
+            for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+              for (int q = 0; q < 8; ++q)
+                // rows 8 (q / 2) + 4 (lane / 32) + 2 (q % 2) and the next: row pair 4 (q / 2) + 2 (lane / 32) + q % 2
+                words[(4 * (q / 2) + (row_lane >> 1) + (q & 1)) * WCOLS + ((fn * 32 + col_lane) ^ half_write ^ ((q & 1) << 2))] =
+                    pack(acc[fm][fn][2 * q], acc[fm][fn][2 * q + 1]);
+          }
 #pragma unroll
           for (int it = 0; it < ITERS; ++it) {
             const int task = it * 64 + lane;
@@ -943,11 +1126,7 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
             c_raw[it][0] = lo.x; c_raw[it][1] = lo.y; c_raw[it][2] = lo.z; c_raw[it][3] = lo.w;
             c_raw[it][4] = hi.x; c_raw[it][5] = hi.y; c_raw[it][6] = hi.z; c_raw[it][7] = hi.w;
           }
-#pragma unroll
-          for (int fn = 0; fn < FN; ++fn)
-#pragma unroll
-            for (int v = 0; v < 16; ++v)
-              scratch[(8 * (v / 4) + row_lane + (v % 4)) * WCOLS + ((fn * 32 + col_lane) ^ half_write ^ ((v & 1) << 2))] = acc[fm][fn][v];
+          store_rows(fm);
 #pragma unroll
           for (int it = 0; it < ITERS; ++it) {
             const int piece = it * 64 + lane;
@@ -998,11 +1177,7 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
             }
             c_raw[it][0] = lo.x; c_raw[it][1] = lo.y; c_raw[it][2] = lo.z; c_raw[it][3] = lo.w;
           }
-#pragma unroll
-          for (int fn = 0; fn < FN; ++fn)
-#pragma unroll
-            for (int v = 0; v < 16; ++v)
-              scratch[(8 * (v / 4) + row_lane + (v % 4)) * WCOLS + ((fn * 32 + col_lane) ^ half_write ^ ((v & 1) << 2))] = acc[fm][fn][v];
+          store_rows(fm);
 #pragma unroll
           for (int it = 0; it < ITERS; ++it) {
             const int piece = it * 64 + lane;
@@ -1033,6 +1208,29 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
     }
   }
   // Direct form (generic variant, or C / D not 16-byte aligned): one element per accumulator register.
+  auto finish_element = [&](int row, int col, float sum) __attribute__((always_inline)) {
+    if (row < row_limit && col < p.n) {
+      const size_t o = (size_t)row * p.n + col;
+      float x = p.alpha * sum;
+      if (p.beta != 0.f) {
+        const float cv = p.c_f16 ? (float)reinterpret_cast<const _Float16*>(p.c)[o]
+                                 : reinterpret_cast<const float*>(p.c)[o];
+        x = x + p.beta * cv;
+      }
+      if (p.d_f16) reinterpret_cast<_Float16*>(d_out)[o] = (_Float16)x;
+      else reinterpret_cast<float*>(d_out)[o] = x;
+    }
+  };
+  if constexpr (M16) {
+#pragma unroll
+    for (int rt = 0; rt < 2 * FM; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < 2 * FN; ++ct)
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          finish_element(row0 + rt * 16 + 4 * (lane >> 4) + v, col0 + ct * 16 + (lane & 15), acc16[rt][ct][v]);
+    return;
+  }
   const int col_lane = lane & 31;
   const int row_lane = 4 * (lane >> 5);
 #pragma unroll
@@ -1043,18 +1241,7 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
       const int col = col0 + fn * 32 + col_lane;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int row = row0 + fm * 32 + 8 * (v / 4) + row_lane + (v % 4);
-        if (row < row_limit && col < p.n) {
-          const size_t o = (size_t)row * p.n + col;
-          float x = p.alpha * acc[fm][fn][v];
-          if (p.beta != 0.f) {
-            const float cv = p.c_f16 ? (float)reinterpret_cast<const _Float16*>(p.c)[o]
-                                     : reinterpret_cast<const float*>(p.c)[o];
-            x = x + p.beta * cv;
-          }
-          if (p.d_f16) reinterpret_cast<_Float16*>(d_out)[o] = (_Float16)x;
-          else reinterpret_cast<float*>(d_out)[o] = x;
-        }
+        finish_element(row0 + fm * 32 + 8 * (v / 4) + row_lane + (v % 4), col, acc[fm][fn][v]);
       }
     }
   }
@@ -1577,13 +1764,13 @@ hipError_t launch_pack(const void* w, void* a, void* e, int m, int k, int prune,
   return hipGetLastError();
 }
 
-template <int WM, int WN, int FM, int FN, bool DMA, bool TOKENS = false, int KG = 1>
+template <int WM, int WN, int FM, int FN, bool DMA, bool TOKENS = false, int KG = 1, bool M16 = false>
 static hipError_t launch_gemm_cfg(GemmArgs args, hipStream_t stream) {
   using TS = TileShape<WM, WN, FM, FN, KG>;
   args.tiles_m = (args.m + TS::BM - 1) / TS::BM;
   args.tiles_n = (args.n + TS::BN - 1) / TS::BN;
   const int lds = DMA ? TS::LDS_BYTES : TS::STAGE_BYTES;
-  auto kern = gemm_kernel<WM, WN, FM, FN, DMA, TOKENS, KG>;
+  auto kern = gemm_kernel<WM, WN, FM, FN, DMA, TOKENS, KG, M16>;
   // the dynamic-LDS limit is a per-device attribute of the kernel; threads that race here set the same value
   static std::atomic<bool> attr_done[64] = {};
   int device = 0;
@@ -1621,6 +1808,7 @@ static hipError_t launch_gemm_pass(GemmArgs args, int tile_config, hipStream_t s
     case kTile64x128: return launch_gemm_cfg<2, 2, 1, 2, true>(args, stream);
     case kTile128x128k2: return launch_gemm_cfg<2, 2, 2, 2, true, false, 2>(args, stream);
     case kTile64x128k2: return launch_gemm_cfg<2, 2, 1, 2, true, false, 2>(args, stream);
+    case kTile512x128m16: return launch_gemm_cfg<4, 1, 4, 4, true, false, 1, true>(args, stream);
     default: return hipErrorInvalidValue;
   }
 }

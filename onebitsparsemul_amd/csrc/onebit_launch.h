@@ -54,7 +54,7 @@ struct SkinnyArgs {
   float* split_ws;
 };
 
-enum TileConfig { kTile512x128 = 0, kTile256x128 = 1, kTile128x128 = 2, kTile256x256 = 3, kTile256x128w = 4, kTile512x128t = 5, kTile128x128s = 6, kTile256x64 = 7, kTile256x256w8 = 8, kTile512x128w8 = 9, kTile256x128w8 = 10, kTile128x128w8 = 11, kTile64x128 = 12, kTile128x128k2 = 13, kTile64x128k2 = 14, kTileAuto = -1 };
+enum TileConfig { kTile512x128 = 0, kTile256x128 = 1, kTile128x128 = 2, kTile256x256 = 3, kTile256x128w = 4, kTile512x128t = 5, kTile128x128s = 6, kTile256x64 = 7, kTile256x256w8 = 8, kTile512x128w8 = 9, kTile256x128w8 = 10, kTile128x128w8 = 11, kTile64x128 = 12, kTile128x128k2 = 13, kTile64x128k2 = 14, kTile512x128m16 = 15, kTileAuto = -1 };
 
 hipError_t launch_prepare(const void* a, const void* e, void* prep, int m, int k, int layout, hipStream_t stream);
 hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream);

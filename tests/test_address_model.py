@@ -19,7 +19,8 @@ LANE = np.arange(64, dtype=np.int64)
 # TileConfig code -> (WM, WN, FM, FN, KG), as in launch_gemm_pass
 TILES = {0: (4, 1, 4, 4, 1), 1: (4, 1, 2, 4, 1), 2: (4, 1, 1, 4, 1), 3: (2, 2, 4, 4, 1), 4: (2, 2, 4, 2, 1),
          5: (2, 2, 8, 2, 1), 6: (2, 2, 2, 2, 1), 7: (2, 2, 4, 1, 1), 8: (2, 4, 4, 2, 1), 9: (4, 2, 4, 2, 1),
-         10: (4, 2, 2, 2, 1), 11: (2, 4, 2, 1, 1), 12: (2, 2, 1, 2, 1), 13: (2, 2, 2, 2, 2), 14: (2, 2, 1, 2, 2)}
+         10: (4, 2, 2, 2, 1), 11: (2, 4, 2, 1, 1), 12: (2, 2, 1, 2, 1), 13: (2, 2, 2, 2, 2), 14: (2, 2, 1, 2, 2),
+         15: (4, 1, 4, 4, 1)}  # 15: tile 0's geometry on the 16x16x64 SMFMAC (same copies, same result region)
 
 
 def prepared_bytes(m, k):

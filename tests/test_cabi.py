@@ -143,9 +143,11 @@ def _default_hooks():
 def test_launch_plan_of_the_benchmark_shapes(_default_hooks):
     """kernel choice of the C ABI (host logic, no GPU): the five benchmark configurations and the cases around them"""
     plan = _native.describe_launch
-    # large squares: 512 x 128 tile on eight wavefronts (code 9), one pass, B read in place
+    # large squares: at least one round of 512 x 128 tiles, which then run on the 16x16x64 SMFMAC with one wavefront per
+    # SIMD (code 15); one pass, B read in place
     for size in (4096, 8192, 16384, 25600):
-        assert plan(size, size, size) == dict(kernel="gemm_kernel", tile=9, splits=1, pad_b=False)
+        assert plan(size, size, size) == dict(kernel="gemm_kernel", tile=15, splits=1, pad_b=False)
+    assert plan(28672, 512, 8192)["tile"] == 15                                                   # 224 tiles: 0.875 of a round
     # a last round of 512 x 128 tiles that would be mostly empty: 256 x 128 on four wavefronts (code 4)
     assert plan(6144, 6144, 6144)["tile"] == 4 and plan(11008, 2048, 4096)["tile"] == 4
     # the prefill shape has one 256 x 128 tile per CU: its eight-wavefront form (code 10)
@@ -174,7 +176,7 @@ def test_launch_plan_of_the_benchmark_shapes(_default_hooks):
     assert plan(65536, 64, 8192)["kernel"] == "gemm_kernel"      # from about 48k rows on the main kernel is faster
     assert plan(4096, 65, 4096)["kernel"] == "gemm_kernel"
     # fewer than 256 tiles of 512 x 128: tile and split from the cost model
-    assert plan(4096, 3072, 4096) == dict(kernel="gemm_kernel", tile=9, splits=1, pad_b=False)    # 192 large tiles
+    assert plan(4096, 3072, 4096) == dict(kernel="gemm_kernel", tile=9, splits=1, pad_b=False)    # 192 large tiles: eight wavefronts
     assert plan(4096, 1536, 4096) == dict(kernel="gemm_kernel", tile=10, splits=1, pad_b=False)   # 192 of 256 x 128
     assert plan(11008, 768, 4096)["tile"] == 9 and plan(28672, 192, 8192)["tile"] == 10
     assert plan(4096, 384, 11008) == dict(kernel="gemm_kernel", tile=13, splits=2, pad_b=False)   # 96 tiles, 43 chunks

@@ -428,7 +428,7 @@ def test_ragged_shapes(m, n, k):
     assert np.array_equal(_run_prepared(a, meta, bi, m, n, k, out_dtype=torch.float32), exact)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15])
 @pytest.mark.parametrize("m,n,k", [(1024, 512, 1024), (576, 264, 192), (2112, 1032, 64)])
 def test_every_tile_configuration(tile, m, n, k):
     _native.set_tile_config(tile)

@@ -36,7 +36,7 @@ def test_random_cases_match_the_oracle(seed):
         beta = float(rng.choice([0.0, 1.0]))
         out_dtype = torch.float32 if rng.random() < 0.5 else torch.float16
         hooks = dict(skinny=bool(rng.random() < 0.8), rows=int(rng.choice([-1, 32, 64, 128])),
-                     split=int(rng.choice([-1, -1, 1, 2, 3, 5])), tile=int(rng.choice([-1, -1, -1] + list(range(15)))),
+                     split=int(rng.choice([-1, -1, 1, 2, 3, 5])), tile=int(rng.choice([-1, -1, -1] + list(range(16)))),
                      pad=bool(rng.random() < 0.8))
         offset = int(rng.choice([0, 0, 1, 4, 8]))  # halves: B 2, 8 or 16 bytes past a 16-byte boundary
         static = bool(rng.random() < 0.4)          # the entry point whose buffers live in the fixed device array
