@@ -119,7 +119,7 @@ const char *onebit_sparse_last_error(void);
 
 /* Tuning / test hooks: force a tile configuration of the main kernel (-1 = automatic) and choose whether
  * shapes with n <= 32 (n <= 64 when m <= 40960) use the split-K kernel (1, default) or the main kernel (0).
- * Tile codes 0-14 are the TileConfig values of csrc/onebit_launch.h (the linear-layer form has 4, 6, 9-14).
+ * Tile codes 0-15 are the TileConfig values of csrc/onebit_launch.h (the linear-layer form has 4, 6, 9-14).
  * These five hooks act on the calling thread only: the calls that thread makes afterwards. */
 void onebit_sparse_set_tile_config(int tile_config);
 void onebit_sparse_set_skinny_enabled(int enabled);

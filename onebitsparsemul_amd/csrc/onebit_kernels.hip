@@ -206,7 +206,7 @@ struct TileShape {
 // XCD-aware tile order. Workgroup b runs on XCD b % 8, so XCD x is given a contiguous range of a tile list
 // that is ordered in blocks of GROUP_M row tiles x 4 column tiles (row tile fastest), blocks running down M inside
 // a strip of 4 column tiles, strips running along N. GROUP_M x 4 = the workgroups resident on one XCD (64 for the
-// four-wavefront tiles, two per CU; 32 for the eight-wavefront tiles), which then form one block: every B column
+// four-wavefront tiles with two workgroups per CU; 32 for the tiles with one per CU), which then form one block: every B column
 // panel it streams is shared by GROUP_M workgroups and every A row panel by 4 in that XCD's L2, and the whole
 // range of one XCD covers few column strips, so B is fetched into few L2s.
 template <int GROUP_M>
@@ -341,7 +341,8 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
   const int wave_in_group = KG == 2 ? wave % (WM * WN) : wave;
   const int wm = wave_in_group / WN, wn = wave_in_group % WN;
   int tile_m, tile_n;
-  tile_of_block<(NW == 8 ? 8 : 16)>(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  // one workgroup per compute unit (eight wavefronts, or four that use all the registers): 32 resident on an XCD
+  tile_of_block<(NW == 8 || FM * FN > 8 ? 8 : 16)>(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
   const int row0 = tile_m * BM + wm * FM * 32;  // first row of this wavefront
   const int n0 = tile_n * BN;                   // first column of the workgroup
   const int col0 = n0 + wn * FN * 32;           // first column of this wavefront

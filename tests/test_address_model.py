@@ -244,7 +244,7 @@ def check_gemm(m, n, k, tile, splits, pad_b, tokens=False, b_aligned=True, d_siz
     if tokens:
         assert k * 256 * 2 < (1 << 32)
     # the workgroup -> tile mapping is a bijection
-    seen = {tile_of_block(b, tiles_m, tiles_n, 8 if NW == 8 else 16) for b in range(tiles_m * tiles_n)}
+    seen = {tile_of_block(b, tiles_m, tiles_n, 8 if NW == 8 or FM * FN > 8 else 16) for b in range(tiles_m * tiles_n)}
     assert seen == {(tm, tn) for tm in range(tiles_m) for tn in range(tiles_n)}
     rb_total = m // 32
     corner_tiles = {(0, 0), (tiles_m - 1, 0), (0, tiles_n - 1), (tiles_m - 1, tiles_n - 1), (tiles_m // 2, tiles_n // 2)}
