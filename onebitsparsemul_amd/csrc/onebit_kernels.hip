@@ -1254,7 +1254,8 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
 // takes the K chunks (of 256) w, w + NW, w + 2 NW, ... Each wavefront stages B rows in a private 8 KiB LDS region
 // as a zero-padded fp16 image of NC columns (NC = 16: the 256 rows of a chunk; NC = 32: 128 rows, two images per
 // chunk; NC = 64: 64 rows, four images, two column fragments), feeds them to SMFMAC through transpose reads (one fragment serves the R row blocks) and keeps a 32x32
-// fp32 partial tile per row block. The prepared operand and the next image are loaded into registers while the
+// fp32 partial tile per row block (NC = 16: two 16x16 tiles, multiplied with v_smfmac_f32_16x16x64_f16, which has no
+// idle columns at sixteen). The prepared operand and the next image are loaded into registers while the
 // current one is multiplied. Wavefronts never wait for one another inside the K loop (LDS operations of one
 // wavefront execute in order). The NW partial tiles of a row block are added through LDS in wavefront order
 // (deterministic; the tiles take the place of the images, as many row blocks per round as fit the 8 KiB) and the
@@ -1269,7 +1270,11 @@ constexpr int kSkinnyRegion = 8192;  // bytes of one B image
 // the image's K range of token t in 16-byte pieces, piece p stored at position p ^ token_swizzle(t) so that lanes
 // which read the same piece of consecutive tokens fall into different banks; a lane's SMFMAC operand is two plain
 // 16-byte reads (K consecutive inside a piece), no transpose.
-enum SkinnyBMode { kSkinnyBFull = 0, kSkinnyB8 = 1, kSkinnyB4 = 2, kSkinnyBScalar = 3, kSkinnyBTokens = 4 };
+// kSkinnyBRun: n = 2 or 4 with B 16-byte aligned. The 256 rows of a chunk are one run of 512 n consecutive bytes,
+// loaded in 16-byte pieces (32 n of them: at most two load instructions per wavefront and chunk, where the row-wise
+// modes issue eight; the split-K kernel's time is set by the number of load instructions it issues) and spread over the image rows
+// by LDS stores of 2 n bytes.
+enum SkinnyBMode { kSkinnyBFull = 0, kSkinnyB8 = 1, kSkinnyB4 = 2, kSkinnyBScalar = 3, kSkinnyBTokens = 4, kSkinnyBRun = 5 };
 
 // 16-byte piece q of the image whose first row is B row k_base: image row q / (NC / 8), columns 8 (q % (NC / 8))
 // ... + 7; zero outside B. Vector modes only.
@@ -1310,10 +1315,14 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   constexpr int TILE_BYTES = kRowBlock * NC * 4;       // one fp32 partial tile
   static_assert(NC == 16 || NC == 32 || NC == 64, "image width");
   static_assert(MODE != kSkinnyB4 || NC == 16, "the 8-byte-row mode is for 16 columns");
+  static_assert(MODE != kSkinnyBRun || NC == 16, "the run mode is for 16 columns");
   // the partial tiles reuse the wavefront's image memory, RT row blocks per round of the final reduction
   constexpr int RT = R * TILE_BYTES <= kSkinnyRegion ? R : kSkinnyRegion / TILE_BYTES;
   static_assert(RT >= 1 && R % RT == 0, "the row blocks must divide into whole reduction rounds");
   constexpr bool TOKENS = MODE == kSkinnyBTokens;
+  // Sixteen columns fill half of the 32x32x32 SMFMAC's result tile; v_smfmac_f32_16x16x64_f16 has no idle half and
+  // multiplies a row block's chunk in half the matrix-pipe time (eight instructions of four passes).
+  constexpr bool M16 = NC == 16;
   constexpr int PPT = IMG_ROWS / 8;                    // token-major image: 16-byte pieces per token row
   constexpr int TPI = 64 / PPT;                        // ... and tokens covered by the 64 pieces of one wavefront load
   constexpr int TOKEN_ROW_BYTES = IMG_ROWS * 2;
@@ -1369,23 +1378,50 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   const uint32_t token_load_step = (uint32_t)TPI * (uint32_t)k_rows * 2u;
   const uint32_t token_store_base =
       (uint32_t)token_lane * TOKEN_ROW_BYTES + (uint32_t)((piece_lane ^ token_swizzle<TOKEN_ROW_BYTES>(token_lane)) << 4);
+  // run mode: piece q = lane + 64 i of the image's run; pieces at or past 32 n are sent outside the descriptor (zero)
+  const uint32_t run_pieces = 32u * (uint32_t)n_cols;
   auto load_b = [&](int k_base, u32x4_t (&v)[8]) __attribute__((always_inline)) {
     if (MODE == kSkinnyBScalar) return;
+    if (MODE == kSkinnyBRun) {
+      const uint32_t run_base = (uint32_t)k_base * (uint32_t)n_cols * 2u;  // the launcher checks k n 2 < 2^32
+      if (k_base + IMG_ROWS <= k_rows) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          if (64u * i < run_pieces)
+            v[i] = buffer_load16(b_buffer, lane + 64u * i < run_pieces ? meta_off + 1024u * i : 0xFFFFFF00u, run_base);
+        return;
+      }
+      // last image of a K that is no multiple of 256 (or an image past the end that is loaded but never multiplied):
+      // pieces inside B as they are, zeros past its end. K is a multiple of 32, so the valid bytes are a multiple of 16 n
+      // and no piece straddles the end.
+      const uint32_t valid_bytes = (uint32_t)rows_valid_of(k_base) * (uint32_t)n_cols * 2u;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        if (64u * i < run_pieces)
+          v[i] = buffer_load16(b_buffer, meta_off + 1024u * i + 16u <= valid_bytes ? run_base + meta_off + 1024u * i : 0xFFFFFF00u, 0);
+      return;
+    }
     if (TOKENS) {
       // offsets at or past n * k * 2 (tokens >= n) fall outside the descriptor and read as zero; K positions at or
       // past k are sent there too (the launcher checks that 64 * k * 2 stays well below 2^32)
       if (k_base + IMG_ROWS <= k_rows) {
         // the image's whole K range exists (wave-uniform test): lane offsets that do not change from image to image
         // plus a scalar offset; the range check looks at the lane offset alone, which is what sends tokens >= n to zero
+        // (load i covers tokens TPI i ... TPI i + TPI - 1: nothing to fetch past the last token)
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-          v[i] = buffer_load16(b_buffer, token_load_base + i * token_load_step, (uint32_t)k_base * 2u);
+        for (int i = 0; i < 8; ++i) {
+          if (TPI * i < n_cols) v[i] = buffer_load16(b_buffer, token_load_base + i * token_load_step, (uint32_t)k_base * 2u);
+          else v[i] = u32x4_t{0, 0, 0, 0};
+        }
         return;
       }
       const bool inside = k_base + 8 * piece_lane < k_rows;
       const uint32_t first = token_load_base + (uint32_t)k_base * 2u;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = buffer_load16(b_buffer, inside ? first + i * token_load_step : 0xFFFFFF00u, 0);
+      for (int i = 0; i < 8; ++i) {
+        if (TPI * i < n_cols) v[i] = buffer_load16(b_buffer, inside ? first + i * token_load_step : 0xFFFFFF00u, 0);
+        else v[i] = u32x4_t{0, 0, 0, 0};
+      }
       return;
     }
     if (MODE == kSkinnyBFull && b_fits && k_base + IMG_ROWS <= k_rows) {
@@ -1431,6 +1467,23 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
       }
       return;
     }
+    if (MODE == kSkinnyBRun) {
+      // piece q holds the n columns of rows 8 q / n ... : 2 n bytes to each row's start; columns n ... 15 keep the zeros the
+      // image was cleared to
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const uint32_t q = lane + 64u * i;
+        if (q >= run_pieces) continue;
+        if (n_cols == 4) {
+          *reinterpret_cast<u32x2_t*>(region + (2 * q) * ROW_BYTES) = u32x2_t{v[i].x, v[i].y};
+          *reinterpret_cast<u32x2_t*>(region + (2 * q + 1) * ROW_BYTES) = u32x2_t{v[i].z, v[i].w};
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) *reinterpret_cast<uint32_t*>(region + (4 * q + j) * ROW_BYTES) = v[i][j];
+        }
+      }
+      return;
+    }
     if (TOKENS) {
       // token = token_lane + TPI i with token_lane < TPI (a power of two): the two terms share no bits, so the swizzle of
       // piece i differs from that of piece 0 by a compile-time XOR
@@ -1450,15 +1503,100 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
     for (int f = 0; f < NF; ++f)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[r][f][v] = 0.f;
+  float4v_t acc16[R][2];  // M16: rows 0-15 and 16-31 of the row block; register v of lane l = row 4 (l / 16) + v, column l % 16
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) acc16[r][h] = float4v_t{0.f, 0.f, 0.f, 0.f};
   const uint32_t one = packed_one_in_vgpr();
-  const int i16 = lane & 15, gb = lane >> 5;
-  // NC == 16: lanes 16-31 and 48-63 would hold columns 16-31: they re-read columns 0-15 and are never stored
+  const int i16 = lane & 15, gb = lane >> 5, g16 = lane >> 4;
+  // (32x32x32 form, NC >= 32; sixteen-column images use the 16x16x64 form further down)
   const int chunk8 = (NC >= 32 ? ((lane & 31) >> 4) * 4 : 0) + (i16 & 3);  // 8-byte piece of the 32-column fragment
   const char* lane_ptr = region + (8 * gb + (i16 >> 2)) * ROW_BYTES + chunk8 * 8;
 
   // token-major image: this lane's token row and swizzle; K step s of the image needs pieces 4 s + gb and 4 s + 2 + gb
   const int token_col = NC >= 32 ? (lane & 31) : i16;
   const uint32_t token_read_base = (uint32_t)token_col * TOKEN_ROW_BYTES + (uint32_t)((gb ^ token_swizzle<TOKEN_ROW_BYTES>(token_col)) << 4);
+  // ---- 16x16x64 form (M16). The instruction's A lane (row l % 16, group g = l / 16) holds eight kept values and their
+  // 16 index bits for 16 consecutive K positions, as a lane of the prepared block does for one K step: lane
+  // (row, half ga) of the block, step s. Which K positions group g stands for is free as long as B agrees, so the
+  // operands are built with one v_permlane16_swap per register pair instead of a gather: swapping the odd 16-lane
+  // rows of metadata register 2 P with the even rows of register 2 P + 1 leaves in the first register, for
+  // block rows 0-15, the groups (ga 0, steps 4 P + {0, 1}), (ga 0, steps 4 P + {2, 3}), (ga 1, steps 4 P + {0, 1}),
+  // (ga 1, steps 4 P + {2, 3}) and in the second register the same for block rows 16-31; ABID picks the even or the
+  // odd step of each pair. Instruction (P, abid) therefore covers K positions 128 P + 32 abid + [0, 32) and
+  // 128 P + 32 abid + 64 + [0, 32) of the chunk: group g positions 128 P + 32 abid + 64 (g % 2) + 16 (g / 2) + [0, 16).
+  // The sign words travel the same way (a register swapped with its own copy) and are shifted by 8 (g % 2) once, after
+  // which the expansion uses compile-time shifts. B lane (column l % 16, group gb) holds instruction K rows
+  // 8 gb + [0, 8) and 32 + 8 gb + [0, 8), i.e. chunk rows base + [0, 8) and base + 16 + [0, 8) with
+  // base = 128 P + 32 abid + 64 (gb / 2) + 8 (gb % 2).
+  struct A16 {
+    uint32_t idx[2][2];   // [row half][P]
+    uint32_t sign[2][2];
+  };
+  const uint32_t sign_shift16 = 8u * (g16 & 1);
+  auto gather16 = [&](const AChunk& a) __attribute__((always_inline)) {
+    A16 t;
+#pragma unroll
+    for (int P = 0; P < 2; ++P) {
+      const auto m = __builtin_amdgcn_permlane16_swap(a.meta[2 * P], a.meta[2 * P + 1], false, false);
+      const uint32_t w = P == 0 ? a.sign.x : a.sign.y;
+      const auto sg = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+      t.idx[0][P] = m[0];
+      t.idx[1][P] = m[1];
+      t.sign[0][P] = sg[0] << sign_shift16;
+      t.sign[1][P] = sg[1] << sign_shift16;
+    }
+    return t;
+  };
+  const char* lane_ptr16 = region + (64 * (g16 >> 1) + 8 * (g16 & 1) + (i16 >> 2)) * ROW_BYTES + (i16 & 3) * 8;
+  const uint32_t token_read_base16 =
+      (uint32_t)i16 * TOKEN_ROW_BYTES + (uint32_t)(((8 * (g16 >> 1) + (g16 & 1)) ^ token_swizzle<TOKEN_ROW_BYTES>(i16)) << 4);
+  // B operand of instruction F = 2 P + abid
+  auto frag16 = [&](int F) __attribute__((always_inline)) {
+    u32x8_t raw;
+    if (TOKENS) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const u32x4_t t = *reinterpret_cast<const u32x4_t*>(
+            region + (token_read_base16 ^ (uint32_t)((16 * (F >> 1) + 4 * (F & 1) + 2 * h) << 4)));
+        raw[4 * h] = t.x; raw[4 * h + 1] = t.y; raw[4 * h + 2] = t.z; raw[4 * h + 3] = t.w;
+      }
+      return __builtin_bit_cast(half16_t, raw);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int row_const = 128 * (F >> 1) + 32 * (F & 1) + 4 * (q & 1) + 16 * (q >> 1);
+      const u32x2_t t = lds_read_tr16(lane_ptr16 + row_const * ROW_BYTES);
+      raw[2 * q] = t.x;
+      raw[2 * q + 1] = t.y;
+    }
+    return __builtin_bit_cast(half16_t, raw);
+  };
+  auto compute16 = [&](const AChunk (&a)[R]) __attribute__((always_inline)) {
+    half16_t bf[4];
+#pragma unroll
+    for (int F = 0; F < 4; ++F) bf[F] = frag16(F);
+    A16 t[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) t[r] = gather16(a[r]);
+#pragma unroll
+    for (int F = 0; F < 4; ++F)
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          u32x4_t av;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) av[q] = ((t[r].sign[h][F >> 1] << (4 * (F & 1) + q)) & 0x80008000u) | one;
+          const half8_t a8 = __builtin_bit_cast(half8_t, av);
+          if ((F & 1) == 0)
+            acc16[r][h] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a8, bf[F], acc16[r][h], (int)t[r].idx[h][F >> 1], 0, 0);
+          else
+            acc16[r][h] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a8, bf[F], acc16[r][h], (int)t[r].idx[h][F >> 1], 0, 1);
+        }
+  };
+
   auto frag = [&](int image_step, int f) __attribute__((always_inline)) {
     u32x8_t raw;
     if (TOKENS) {
@@ -1481,6 +1619,10 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   };
   // the SMFMACs of image SUB_INDEX of a chunk: steps SUB_INDEX * IMG_STEPS ... + IMG_STEPS - 1
   auto compute = [&](const AChunk (&a)[R], auto sub_tag) __attribute__((always_inline)) {
+    if constexpr (M16) {
+      compute16(a);
+      return;
+    }
     constexpr int FIRST_STEP = decltype(sub_tag)::value * IMG_STEPS;
     // Fragments are read in groups of FG K steps (4 FG transpose reads per column fragment) into one of two register
     // sets: while the SMFMACs of a group run, the reads of the next group are already in flight, so only the first
@@ -1534,7 +1676,7 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
 
   // sixteen wavefronts leave 128 registers each: no room to hold the next image (32 registers) during the SMFMACs
   constexpr bool kPrefetchB = NW <= 8 && MODE != kSkinnyBScalar;
-  if (MODE == kSkinnyBScalar) {
+  if (MODE == kSkinnyBScalar || MODE == kSkinnyBRun) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4_t*>(region + (lane + i * 64) * 16) = u32x4_t{0, 0, 0, 0};
   }
@@ -1604,7 +1746,19 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
     {
       float* tile = reinterpret_cast<float*>(region);
       const int col = lane & 31;
-      if (col < NC) {
+      if (M16) {
+#pragma unroll
+        for (int rr = 0; rr < RT; ++rr)
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+              const int row = 16 * h + 4 * g16 + v;
+              const float value = acc16[round * RT + rr][h][v];
+              if (TOKENS) tile[i16 * ROUND_ROWS + ((rr * 32 + row) ^ i16)] = value;
+              else tile[(rr * 32 + row) * NC + i16] = value;
+            }
+      } else if (col < NC) {
 #pragma unroll
         for (int rr = 0; rr < RT; ++rr)
 #pragma unroll
@@ -1634,6 +1788,11 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
           if (p.bias) sum += p.bias_f16 ? (float)reinterpret_cast<const _Float16*>(p.bias)[row]
                                         : reinterpret_cast<const float*>(p.bias)[row];
           const size_t o = (size_t)token * p.m + row;
+          // a B of one column is a token-major x of one token and its result column is y: the launcher sends such calls
+          // here with their alpha, beta and C (element o of C in both layouts); the linear layer passes 1, 0, null
+          sum = p.alpha * sum;
+          if (p.beta != 0.f)
+            sum = sum + p.beta * (p.c_f16 ? (float)reinterpret_cast<const _Float16*>(p.c)[o] : reinterpret_cast<const float*>(p.c)[o]);
           if (p.d_f16) reinterpret_cast<_Float16*>(d_out)[o] = (_Float16)sum;
           else reinterpret_cast<float*>(d_out)[o] = sum;
         }
@@ -1913,6 +2072,11 @@ static hipError_t launch_skinny_cfg(const SkinnyArgs& args, hipStream_t stream) 
   }
   if (args.n == 16 && (address & 15) == 0) return launch_skinny_mode<NW, R, kSkinnyBFull, 16>(args, stream);
   if (args.n == 8 && (address & 15) == 0) return launch_skinny_mode<NW, R, kSkinnyB8, 16>(args, stream);
+  // one column: B is a token-major x of one token and D is its y (same memory in both layouts)
+  if (args.n == 1 && (address & 15) == 0 && (size_t)args.k * 64 * 2 < 0xFFFFFF00u)
+    return launch_skinny_mode<NW, R, kSkinnyBTokens, 16>(args, stream);
+  if ((args.n == 2 || args.n == 4) && (address & 15) == 0 && (size_t)args.k * args.n * 2 < 0xFFFFFF00u)
+    return launch_skinny_mode<NW, R, kSkinnyBRun, 16>(args, stream);
   if (args.n == 4 && (address & 7) == 0) return launch_skinny_mode<NW, R, kSkinnyB4, 16>(args, stream);
   return launch_skinny_mode<NW, R, kSkinnyBScalar, 16>(args, stream);
 }

@@ -330,7 +330,7 @@ def test_split_k_kernel_long_k(m, k, ns):
 
 @pytest.mark.parametrize("rows,splits", [(32, 2), (64, 3), (64, 16), (128, 4), (-1, -1)])
 @pytest.mark.parametrize("m,n,k", [(256, 16, 8192), (192, 5, 4128), (320, 32, 12320), (128, 40, 8224), (1024, 64, 16384),
-                                   (4096, 16, 16384)])
+                                   (4096, 16, 16384), (256, 1, 8224), (192, 2, 8192), (320, 4, 4128)])
 def test_split_k_kernel_with_k_split_over_workgroups(rows, splits, m, n, k):
     """the split-K kernel with K split over workgroups as well (partial sums + ordered reduction): forced split counts
     that do and do not divide the chunk count, splits with fewer chunks than wavefronts, K tails, every image width,
@@ -439,6 +439,38 @@ def test_every_tile_configuration(tile, m, n, k):
     exact = oracle.host_gemm(dense, bi.numpy(), c=c.numpy(), alpha=2.0, beta=-1.0, d_dtype=oracle.F32)
     got = _run_prepared(a, meta, bi, m, n, k, c=c, alpha=2.0, beta=-1.0, out_dtype=torch.float32)
     assert np.array_equal(got, exact)
+
+
+@pytest.mark.parametrize("rows", [32, 64, 128])
+@pytest.mark.parametrize("offset", [0, 4, 1])  # B 16-byte aligned, 8-byte aligned, 2-byte aligned
+@pytest.mark.parametrize("m,n,k", [(320, 1, 4128), (192, 1, 800), (2240, 1, 8224), (64, 1, 256), (320, 2, 4128),
+                                   (192, 2, 800), (1088, 2, 2048), (320, 4, 4128), (192, 4, 800), (2240, 4, 8224)])
+def test_split_k_kernel_few_columns(rows, offset, m, n, k):
+    """n = 1 (B read as a token-major x of one token, with the call's alpha, beta and C), n = 2 and 4 (a chunk's rows read
+    as one run of 16-byte pieces) and what the same shapes fall back to when B is not 16-byte aligned; K tails, chunk
+    counts that do not divide among the wavefronts, C and D in one buffer"""
+    _native.set_skinny_rows(rows)
+    a, meta = synthetic.make_weight(m, k, seed=rows + m + k + n)
+    dense = oracle.decompress_operands(a.numpy(), meta.numpy(), m, k)
+    bi = synthetic.make_b(k, n, seed=n, kind="int")
+    ci = synthetic.make_c(m, n, seed=n + 1, dtype=torch.float32).round()
+    exact = oracle.host_gemm(dense, bi.numpy(), c=ci.numpy(), alpha=2.0, beta=1.0, d_dtype=oracle.F32, acc="f32")
+    ad, md = _gpu(a, meta)
+    prep = _native.prepare(ad, md, m, k)
+    storage = torch.zeros(k * n + 16, dtype=torch.float16, device="cuda")
+    bd = storage[offset:offset + k * n].view(k, n)
+    bd.copy_(bi.cuda())
+    assert bd.data_ptr() % 16 == (2 * offset) % 16 and bd.is_contiguous()
+    d = ci.cuda()  # C and D share the buffer
+    _native.matmul_prepared(prep, bd, d, m, n, k, c=d, alpha=2.0, beta=1.0)
+    torch.cuda.synchronize()
+    assert np.array_equal(d.cpu().numpy(), exact)
+    b = synthetic.make_b(k, n, seed=n + 50, kind="normal")
+    bd.copy_(b.cuda())
+    d16 = torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda")
+    _native.matmul_prepared(prep, bd, d16, m, n, k)
+    torch.cuda.synchronize()
+    _assert_close(d16.cpu().numpy(), oracle.blas_matmul(dense, b.numpy()))
 
 
 @pytest.mark.parametrize("n", [72, 64, 32, 16, 8])  # main kernel's element-copy variant; split-K kernel's element mode
