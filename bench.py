@@ -26,9 +26,9 @@ HBM_PEAK_GBS = 8000.0
 # HBM-side bytes per launch of the dominant kernel, from two rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE), each
 # scaled by what the same counter reads for an elementwise copy kernel over 256 MiB (x2.000 and x1.000): see
 # profiles/hbm_traffic_counters.txt. Only the workloads it was measured on have a figure.
-MEASURED_TRAFFIC_BYTES = {"square:8192": (229542.5 * 2.000 + 131072.0 * 1.000) * 1024,
-                          "prefill": (30824.0 * 2.000 + 16384.0 * 1.000) * 1024,
-                          "decode:11008x4096x16": (4709.6 * 2.000 + 344.0 * 1.000) * 1024}
+MEASURED_TRAFFIC_BYTES = {"square:8192": (229619.5 * 2.000 + 131072.0 * 1.000) * 1024,
+                          "prefill": (30840.0 * 2.000 + 16384.0 * 1.000) * 1024,
+                          "decode:11008x4096x16": (4709.0 * 2.000 + 344.0 * 1.000) * 1024}
 
 
 def parse_workload(text):

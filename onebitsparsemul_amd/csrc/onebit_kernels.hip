@@ -180,8 +180,10 @@ constexpr int kStages = 4;  // LDS ring; one prepared-operand chunk (256 K) = on
 
 template <int BN>
 __device__ __forceinline__ int chunk_swizzle(int row) {
-  // 16-byte chunk index XOR; rows r..r+3 must land in four different 64-byte bank groups.
-  return (BN >= 128) ? ((row & 3) << 2) : (((row >> 1) & 1) << 2);
+  // 16-byte chunk index XOR; rows r..r+3 must land in four different 64-byte bank groups. Bit 3 of the row swaps the
+  // 32-byte halves of a group: the 16x16x64 form's lanes 0-15 and 16-31 read 32 bytes each of rows r..r+3 and
+  // r+8..r+11 in one pass (the 32x32x32 form reads whole 64-byte groups and does not notice).
+  return (BN >= 128) ? (((row & 3) << 2) | (((row >> 3) & 1) << 1)) : (((row >> 1) & 1) << 2);
 }
 
 // KG = 2: two groups of WM x WN wavefronts cover the same tile; group g multiplies K step g of every 64-row stage,

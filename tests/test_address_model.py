@@ -267,7 +267,7 @@ def check_gemm(m, n, k, tile, splits, pad_b, tokens=False, b_aligned=True, d_siz
                             stage_stride, stage0 = STAGE_K * 2, n0 * k * 2
                         else:
                             row, pc = slot // CH, slot % CH
-                            sw = ((row & 3) << 2) if BN >= 128 else (((row >> 1) & 1) << 2)
+                            sw = (((row & 3) << 2) | (((row >> 3) & 1) << 1)) if BN >= 128 else (((row >> 1) & 1) << 2)
                             lc = pc ^ sw
                             col = np.where(n0 + 8 * lc >= ldb, 0, 8 * lc)
                             b_off = (row * ldb + col) * 2
