@@ -1713,10 +1713,14 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   if (!short_k) load_a(first, a_cur);
   for (int kc = short_k ? kc_end : first; kc < kc_end; kc += NW) {
     const int k_base = kc * kChunkK;
+    // this wavefront has another chunk after this one (wave-uniform): only then is the next chunk requested; a load
+    // past the last chunk would be one more instruction for the memory pipeline, a third of them when a wavefront
+    // has two or three chunks
+    const bool more = kc + NW < kc_end;
     if (!kPrefetchB) load_b(k_base, breg);
     store_b(k_base, breg);  // after the previous image's fragment reads: LDS operations of a wavefront execute in order
-    if (kPrefetchB) load_b(SUB > 1 ? k_base + IMG_ROWS : k_base + NW * kChunkK, breg);
-    load_a(kc + NW, a_next);
+    if (kPrefetchB && (SUB > 1 || more)) load_b(SUB > 1 ? k_base + IMG_ROWS : k_base + NW * kChunkK, breg);
+    if (more) load_a(kc + NW, a_next);
     compute(a_cur, std::integral_constant<int, 0>{});
     // the chunk's further images (SUB - 1 of them)
     auto further = [&](auto sub_tag) __attribute__((always_inline)) {
@@ -1728,7 +1732,7 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
           load_b(image_base, breg);
         }
         store_b(image_base, breg);
-        if (kPrefetchB) load_b(S + 1 < SUB ? image_base + IMG_ROWS : k_base + NW * kChunkK, breg);
+        if (kPrefetchB && (S + 1 < SUB || more)) load_b(S + 1 < SUB ? image_base + IMG_ROWS : k_base + NW * kChunkK, breg);
         compute(a_cur, sub_tag);
       }
     };
