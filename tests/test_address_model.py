@@ -70,6 +70,10 @@ def skinny_variant(n, rows, b_aligned=True, tokens=False):
         r = min(r, 2)
     if tokens:
         mode = "tokens"
+    elif n == 1 and b_aligned:
+        mode = "tokens"   # a k x 1 B is a token-major x of one token
+    elif n in (2, 4) and b_aligned:
+        mode = "run"      # a chunk's 256 rows as one run of 16-byte pieces
     elif n == nc and b_aligned:
         mode = "full"
     elif nc > 16 and n % 8 == 0 and b_aligned:
@@ -95,8 +99,10 @@ def check_skinny(m, n, k, rows, tokens=False, b_aligned=True, d_size=2, splits=1
     splits = (kc_total + cps - 1) // cps
     assert (splits - 1) * cps < kc_total  # the launcher's check: no empty split
     b_fits = b_size < (1 << 32)
-    if tokens:
+    if mode == "tokens":
         assert k * 64 * 2 < 0xFFFFFF00  # the launcher's check
+    if mode == "run":
+        assert k * n * 2 < 0xFFFFFF00   # the launcher's check
     for wg, split in [(g, sp) for g in sorted({0, 1, grid // 2, grid - 1} & set(range(grid)))
                       for sp in sorted({0, splits // 2, splits - 1})]:
         rb_first = wg * R
@@ -110,10 +116,11 @@ def check_skinny(m, n, k, rows, tokens=False, b_aligned=True, d_size=2, splits=1
             if short_k:
                 chunks += [first, first + nw]
             else:
-                chunks.append(first)
+                chunks.append(first)   # requested before the loop (clamped to the last chunk when past it)
                 kc = first
                 while kc < kc_end:
-                    chunks.append(kc + nw)
+                    if kc + nw < kc_end:
+                        chunks.append(kc + nw)
                     kc += nw
             for r in range(R):
                 rb = min(rb_first + r, rb_total - 1)
@@ -135,8 +142,8 @@ def check_skinny(m, n, k, rows, tokens=False, b_aligned=True, d_size=2, splits=1
                 while kc < kc_end:
                     for s in range(sub):
                         k_bases.append(kc * CHUNK_K + s * img_rows)
-                    if prefetch_b:
-                        k_bases.append(kc * CHUNK_K + nw * CHUNK_K)  # the next chunk's first image, possibly past K
+                    if prefetch_b and kc + nw < kc_end:
+                        k_bases.append(kc * CHUNK_K + nw * CHUNK_K)  # the next chunk's first image
                     kc += nw
             for k_base in k_bases:
                 rows_valid = min(max(k - k_base, 0), img_rows)
@@ -147,6 +154,8 @@ def check_skinny(m, n, k, rows, tokens=False, b_aligned=True, d_size=2, splits=1
                     tpi = 64 // ppt
                     piece_lane, token_lane = LANE % ppt, LANE // ppt
                     for i in range(8):
+                        if tpi * i >= n:
+                            continue  # token groups past the last token are not requested
                         if k_base + img_rows <= k:
                             lane_off = (token_lane * k + 8 * piece_lane) * 2 + i * tpi * k * 2
                             scalar_off = k_base * 2
@@ -161,6 +170,25 @@ def check_skinny(m, n, k, rows, tokens=False, b_aligned=True, d_size=2, splits=1
                         inside(lane_off[accessed] + scalar_off, 16, b_size, "split-K kernel: x rows")
                     continue
                 q_all = LANE[None, :] + 64 * np.arange(8)[:, None]
+                if mode == "run":
+                    # raw buffer loads of 16-byte pieces q = lane + 64 i < 32 n of the run that starts at k_base * n * 2
+                    pieces = 32 * n
+                    for i in range(2):
+                        if 64 * i >= pieces:
+                            continue
+                        at = LANE * 16 + 1024 * i
+                        if k_base + img_rows <= k:
+                            lane_off = np.where(LANE + 64 * i < pieces, at, 0xFFFFFF00)
+                            scalar_off = k_base * n * 2
+                        else:
+                            valid_bytes = rows_valid * n * 2
+                            assert valid_bytes % 16 == 0  # K is a multiple of 32: no piece straddles the end of B
+                            lane_off = np.where(at + 16 <= valid_bytes, k_base * n * 2 + at, 0xFFFFFF00)
+                            scalar_off = 0
+                        accessed = lane_off + 16 <= b_size  # the descriptor's range check looks at the lane offset alone
+                        assert not accessed[lane_off == 0xFFFFFF00].any()
+                        inside(lane_off[accessed] + scalar_off, 16, b_size, "split-K kernel: B run pieces")
+                    continue
                 if mode == "full":
                     if b_fits and k_base + img_rows <= k:
                         inside(k_base * nc * 2 + LANE[None, :] * 16 + 1024 * np.arange(8)[:, None], 16, b_size,
@@ -189,7 +217,7 @@ def check_skinny(m, n, k, rows, tokens=False, b_aligned=True, d_size=2, splits=1
         elem = 4 if splits > 1 else d_size          # a split writes fp32 partial sums to its slice of the workspace
         slice0 = split * m * n * elem if splits > 1 else 0
         total = splits * m * n * elem
-        if tokens:
+        if mode == "tokens":  # (one column: the same element in both layouts)
             inside(slice0 + (cols[None, :] * m + rows_out[:, None]) * elem, elem, total, "split-K kernel: y")
         else:
             inside(slice0 + (rows_out[:, None] * n + cols[None, :]) * elem, elem, total, "split-K kernel: D")
@@ -384,7 +412,9 @@ def test_benchmark_configurations(hooks, m, n, k):
                                              (256, 264, 512, False), (1024, 203, 4128, True), (128, 1000, 4128, True),
                                              (28672, 40, 512, True), (20480, 64, 1024, True), (4096, 384, 11008, True),
                                              (64, 72, 64, False), (2112, 1032, 64, True), (4096, 16, 16384, True),
-                                             (2048, 33, 28672, True), (11008, 32, 28672, True), (192, 5, 12320, True)])
+                                             (2048, 33, 28672, True), (11008, 32, 28672, True), (192, 5, 12320, True),
+                                             (320, 2, 4128, True), (320, 4, 4128, True), (2240, 1, 8224, True),
+                                             (192, 4, 800, False), (192, 2, 12320, True)])
 def test_ragged_and_split_shapes(hooks, m, n, k, b_aligned):
     for rows in (-1, 32, 64, 128):
         _native.set_skinny_rows(rows)
