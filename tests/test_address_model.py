@@ -555,3 +555,54 @@ def test_epilogue_scratch_swizzle_avoids_bank_conflicts():
             sw = ((r & 1) << 2) ^ (((r >> 2) & 1) * 32)
             banks += [(r * wcols + (c8 ^ sw) + j) % 64 for j in range(4)]
         assert len(set(banks)) == 64
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# the split-K kernel's 16x16x64 form: which K positions of a chunk each lane group of an instruction multiplies, on
+# the A side (prepared block lanes after v_permlane16_swap) and on the B side (rows of the image a lane reads)
+# ---------------------------------------------------------------------------------------------------------------
+def _permlane16_swap(x, y):
+    """v_permlane16_swap x, y: the odd 16-lane rows of x trade places with the even rows of y"""
+    x, y = x.copy(), y.copy()
+    for row in (0, 2):
+        lo, hi = slice(16 * row, 16 * row + 16), slice(16 * (row + 1), 16 * (row + 2))
+        x[hi], y[lo] = y[lo].copy(), x[hi].copy()
+    return x, y
+
+
+def test_split_k_16x16x64_operands_agree_on_k():
+    lane = np.arange(64)
+    # lane of the prepared block: row lane % 32, half ga = lane // 32 of each 32-wide K step; metadata register d
+    # holds steps 2 d (low half word, ABID 0) and 2 d + 1 (high, ABID 1); the value tracked here is (lane, register)
+    src = {d: lane * 8 + d for d in range(4)}
+    for P in range(2):
+        first, second = _permlane16_swap(src[2 * P], src[2 * P + 1])
+        for half, reg in enumerate((first, second)):          # operands of block rows 0-15 and 16-31
+            src_lane, src_reg = reg // 8, reg % 8
+            assert np.array_equal(src_lane % 32, 16 * half + lane % 16)  # every lane group holds its own row l % 16
+            ga = src_lane // 32
+            for abid in range(2):
+                step = 2 * src_reg + abid
+                a_first_k = 32 * step + 16 * ga            # the lane's 16 consecutive K positions of the chunk
+                # the instruction pairs A group g, position j with B group (16 g + j) % 32 // 8, slot
+                # 8 ((16 g + j) // 32) + (16 g + j) % 8; a B lane of group gb reads image rows
+                # base + {0..7} (slots 0-7) and base + 16 + {0..7} (slots 8-15)
+                for g in range(4):
+                    first_k = a_first_k[16 * g]
+                    assert (a_first_k[16 * g:16 * g + 16] == first_k).all()
+                    for j in range(16):
+                        ik = 16 * g + j
+                        gb, slot = (ik % 32) // 8, 8 * (ik // 32) + ik % 8
+                        base = 128 * P + 32 * abid + 64 * (gb >> 1) + 8 * (gb & 1)
+                        assert base + slot % 8 + 16 * (slot // 8) == first_k + j
+                # sign bits: register q of step s uses shift 4 (s % 4) + q of the lane's word for steps 4 P ... 4 P + 3;
+                # the kernel shifts by 8 (g % 2) once and then by 4 abid + q
+                g_of_lane = lane // 16
+                assert np.array_equal(4 * (step % 4), 8 * (g_of_lane % 2) + 4 * abid)
+                assert (step // 4 == P).all()
+    # the sign words travel like the metadata: a register swapped with its own copy puts the word of block lane
+    # (row, ga) in lane groups g = 2 ga and 2 ga + 1 of the half that holds the row
+    first, second = _permlane16_swap(lane.copy(), lane.copy())
+    for half, reg in enumerate((first, second)):
+        assert np.array_equal(reg % 32, 16 * half + lane % 16)
+        assert np.array_equal(reg // 32, lane // 32)
