@@ -96,7 +96,7 @@ def time_graph(fn, launches, warmup=20):
     return start.elapsed_time(stop) / launches * 1e-3
 
 
-def run_gemm(w, steps, warmup):
+def make_gemm(w):
     import torch
     from onebitsparsemul_amd import _native, synthetic
     m, n, k = w["m"], w["n"], w["k"]
@@ -106,10 +106,7 @@ def run_gemm(w, steps, warmup):
     prep = _native.prepare(a, meta, m, k)
     d = torch.empty((m, n), dtype=torch.float16, device="cuda")
     fn = lambda i: _native.matmul_prepared(prep, b, d, m, n, k, c=c, alpha=w["alpha"], beta=w["beta"])
-    kernel_s, wall_s = time_launches(fn, steps, warmup)
-    # launches shorter than the host's launch interval: also time them inside a HIP graph
-    graph_s = time_graph(fn, max(steps, 200)) if 2.0 * m * n * k < 2e11 else None
-    return kernel_s, wall_s, (a, meta, b, d), graph_s, fn
+    return (a, meta, b, d), fn
 
 
 def run_decode_rotating(m, k, n, launches=2000, copies=None):
@@ -261,8 +258,20 @@ def main():
         torch.neg(src, out=dst)
         torch.cuda.synchronize()
         del src, dst
-    kernel_s, wall_s, operands, graph_s, fn = run_gemm(w, args.steps, args.warmup)
-    tflops = 2.0 * m * n * k / kernel_s / 1e12
+    operands, fn = make_gemm(w)
+    flops = 2.0 * m * n * k
+    # Order of the legs. After idle the GPU's power management overshoots: it starts at full clock, throttles below the
+    # sustained point within ~3 ms and recovers over the next ~25 ms (8192^3: launches 4-60 after idle run up to 25 %
+    # slower than launch 2 and than every launch from the 60th on). A window of 5 warm-ups + 20 launches taken right
+    # after idle lies inside that dip and measures the transient, not the kernel. So the sustained leg (>= 150 ms of
+    # back-to-back launches, then a HIP-graph timing) runs first and the W warm-ups + K timed launches of the command
+    # line follow it without a pause: `value` is the steady-state rate. `after_idle` repeats exactly the same W + K
+    # sequence after 3 s of idle, i.e. what `value` would be without the preceding load.
+    sustained = None if args.no_sustained else sustained_rate(fn, flops)
+    kernel_s, wall_s = time_launches(fn, args.steps, args.warmup)
+    # launches shorter than the host's launch interval: also time them inside a HIP graph
+    graph_s = time_graph(fn, max(args.steps, 200)) if flops < 2e11 else None
+    tflops = flops / kernel_s / 1e12
     line = dict(
         metric="dense_equiv_tflops", value=tflops, unit="TFLOP/s", n_gpus=1, steps=args.steps, warmup=args.warmup,
         ms_per_step=kernel_s * 1e3, higher_is_better=True, scaling="weak", vs_baseline=None, dtype="f16",
@@ -274,12 +283,20 @@ def main():
                       note="dense-equivalent FLOPs 2MNK against the fp16 SMFMAC rate (2 x the dense fp16 MFMA peak "
                            f"{DENSE_F16_PEAK_TFLOPS:.1f}); the same fraction as executed FLOPs MNK against the dense peak",
                       hbm_gbps_algorithmic=algorithmic_bytes(m, n, k, w["beta"]) / kernel_s / 1e9),
-        wall_ms_per_step=wall_s * 1e3)
-    if not args.no_sustained:
-        line["sustained"] = sustained_rate(fn, 2.0 * m * n * k)
+        wall_ms_per_step=wall_s * 1e3,
+        timing="W warm-ups and K timed launches (HIP events on the launch stream) directly after the sustained leg: "
+               "steady-state clock" if sustained else "W warm-ups and K timed launches from idle")
+    if sustained:
+        line["sustained"] = sustained
+        time.sleep(3.0)
+        idle_s, _ = time_launches(fn, args.steps, args.warmup)
+        line["after_idle"] = dict(ms_per_step=idle_s * 1e3, tflops=flops / idle_s / 1e12,
+                                  frac=flops / idle_s / 1e12 / SMFMAC_PEAK_TFLOPS,
+                                  note="the same W warm-ups + K timed launches after 3 s of idle: the window then lies in "
+                                       "the power management's dip that follows the first launches after idle")
     if graph_s is not None:
         line["graph_ms_per_step"] = graph_s * 1e3  # the same launch inside a HIP graph: no host launch interval
-        line["graph_tflops"] = 2.0 * m * n * k / graph_s / 1e12
+        line["graph_tflops"] = flops / graph_s / 1e12
     from onebitsparsemul_amd import _native
     cus, khz = _native.device_info()
     line["device"] = dict(name=torch.cuda.get_device_name(0), compute_units=cus, clock_mhz=khz / 1e3,
@@ -287,11 +304,21 @@ def main():
                           note="peak = CUs x clock x 4096 dense fp16 FLOP/clk/CU x 2 (sparse); roofline.peak uses the "
                                "published 256 CUs x 2.4 GHz")
     if not args.no_ceiling:
-        # register-only SMFMAC loops: what the chip sustains under matrix load, which depends on the operand values
-        line["smfmac_register_loop_tflops"] = dict(
-            benchmark_distribution=max(_native.measure_smfmac_rate(True, 50000) for _ in range(4)),
-            constant_operands=max(_native.measure_smfmac_rate(False, 50000) for _ in range(4)),
+        # register-only SMFMAC loops: what the chip sustains under matrix load, which depends on the operand values and
+        # on the instruction (m32: v_smfmac_f32_32x32x32_f16, the eight-wavefront tiles; m16: v_smfmac_f32_16x16x64_f16,
+        # the default large tile)
+        rate = _native.measure_smfmac_rate
+        loops = dict(
+            m32_benchmark_distribution=max(rate(True, 50000, _native.SMFMAC_32X32X32) for _ in range(4)),
+            m32_constant_operands=max(rate(False, 50000, _native.SMFMAC_32X32X32) for _ in range(4)),
+            m16_benchmark_distribution=max(rate(True, 100000, _native.SMFMAC_16X16X64) for _ in range(4)),
+            m16_constant_operands=max(rate(False, 100000, _native.SMFMAC_16X16X64) for _ in range(4)),
             note="no LDS or global memory in the loop; the gap to the nominal peak is clock throttling under load")
+        line["smfmac_register_loop_tflops"] = loops
+        tile = _native.describe_launch(m, n, k, compute_units=None).get("tile")
+        ceiling = loops["m16_benchmark_distribution"] if tile == 15 else loops["m32_benchmark_distribution"]
+        line["roofline"]["frac_of_register_loop"] = tflops / ceiling
+        line["roofline"]["register_loop"] = "m16_benchmark_distribution" if tile == 15 else "m32_benchmark_distribution"
     if not args.no_decode:
         line["decode_n16"] = run_decode_rotating(11008, 4096, 16)
         # the same kernel family where the weight is large enough for bandwidth, not latency, to set the time

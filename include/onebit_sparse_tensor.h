@@ -85,10 +85,13 @@ int onebit_sparse_matmul_prepared(const void *prepared, const void *b, const voi
  * aligned): in a fixed array of ONEBIT_STATIC_SCRATCH_BYTES bytes that is part of the library's device code, of
  * which every GPU the library runs on holds one copy until the process ends. The call never calls hipMalloc, hipFree
  * or any allocating routine. A shape whose buffers do not fit is refused with ONEBIT_ERR_ARGUMENT and a message
- * that names the sizes (onebit_sparse_describe_launch tells which shapes need buffers: plan[2] > 1 or plan[3] = 1).
+ * that names the sizes (onebit_sparse_describe_launch of the tuning header tells which shapes need buffers: plan[2] > 1 or plan[3] = 1).
  * The buffers are written in full by the call's own kernels before they are read, so the contents a previous call
  * left behind do no harm; but every call on one GPU uses the same array, so two such calls that overlap in time on
  * one GPU (different streams, or different threads) race. Calls on one stream are ordered and safe.
+ * Cost: the array is part of the library's code object, so every process that loads libonebitmul.so holds
+ * ONEBIT_STATIC_SCRATCH_BYTES (64 MiB) of device memory on each GPU it uses the library on, from the first call of any
+ * entry point on that GPU until the process ends, whether or not it ever calls this one.
  */
 #define ONEBIT_STATIC_SCRATCH_BYTES (64u << 20)
 int onebit_sparse_matmul_prepared_static(const void *prepared, const void *b, const void *c, void *d, int m, int n,
@@ -117,26 +120,6 @@ int onebit_sparse_pack(const void *weight, int m, int k, int prune, void *a, voi
 /* Message of the last failure on the calling thread ("" if none). Host pointer, valid until the next call. */
 const char *onebit_sparse_last_error(void);
 
-/* Tuning / test hooks: force a tile configuration of the main kernel (-1 = automatic) and choose whether
- * shapes with n <= 32 (n <= 64 when m <= 40960) use the split-K kernel (1, default) or the main kernel (0).
- * Tile codes 0-15 are the TileConfig values of csrc/onebit_launch.h (the linear-layer form has 4, 6, 9-14).
- * These five hooks act on the calling thread only: the calls that thread makes afterwards. */
-void onebit_sparse_set_tile_config(int tile_config);
-void onebit_sparse_set_skinny_enabled(int enabled);
-/* Weight rows one workgroup of the split-K kernel covers: 32, 64 or 128; <= 0 = automatic. */
-void onebit_sparse_set_skinny_rows(int rows);
-/* K splits over workgroups, of the main kernel and of the split-K kernel (which also splits K among the wavefronts
- * of a workgroup): 1 = never split, N > 1 = N splits (at most one per 256 of K), <= 0 = automatic (few tiles or row
- * groups and a long K). A split call writes fp32 partial sums to a library-owned buffer kept per
- * device and stream (grown with hipMalloc on first use: warm up before capturing the call in a HIP graph) and adds
- * them in split order, so results do not depend on timing. */
-void onebit_sparse_set_split_k(int splits);
-/* B whose rows are not 16-byte aligned (n % 8 != 0 or an unaligned base) and n beyond the split-K kernel's range:
- * 1 (default) = the main kernel reads a copy of B with rows padded to a multiple of 8 columns, made by one extra
- * pass into a library-owned buffer kept per device and stream (same rules as the K-split buffer); 0 = the main
- * kernel's element-copy variant reads B in place (much slower; always used when k * n < 65536). */
-void onebit_sparse_set_pad_b(int enabled);
-
 /* Opt-in cache for callers of the one-call entry points (onebit_sparse_matmul, onebit_sparse_matmul_ex) whose
  * weights do not change, which is inference: with entries > 0 the library keeps the reordered copy of up to that
  * many weights per device, keyed by (a, e, m, k, meta_layout), in its own device memory, and a call with a known
@@ -154,23 +137,6 @@ int onebit_sparse_clear_weight_cache(void);
  * HIP graphs captured earlier must not be replayed afterwards. No counterpart in the reference (its launcher allocates
  * and frees a workspace on every call, csrc/kernel_lib.cu:73-76). */
 int onebit_sparse_release_buffers(void);
-
-/* Diagnostic, no counterpart in the reference, host-only (touches no GPU): what a prepared call of this shape would
- * launch under the calling thread's hooks on a GPU with 256 compute units (calls plan for the device they run on). plan[0] = 1 for the split-K kernel (n <= 64), 0 for the main kernel; plan[1] =
- * weight rows per workgroup (split-K kernel) or the tile code (main kernel); plan[2] = K splits over workgroups
- * (1 = none); plan[3] = 1 if B is read through a padded copy. */
-int onebit_sparse_describe_launch(int m, int n, int k, int b_16_byte_aligned, int *plan);
-
-/* Diagnostic, no counterpart in the reference: sustained rate of v_smfmac_f32_32x32x32_f16 in a register-only
- * loop on the current device (one wavefront per SIMD, `iterations` x 16 instructions each), in dense-equivalent
- * TFLOP/s. random_operands = 1 uses +-1 values, N(0,1) fp16 B values and random 2:4 indices (the benchmark's
- * distribution), 0 uses constants. The clock the GPU sustains under matrix load depends on the operand values, so
- * this is the practical ceiling next to the nominal peak. Allocates and frees its own device buffers; synchronous. */
-int onebit_sparse_measure_smfmac_rate(int random_operands, int iterations, double *dense_equiv_tflops);
-
-/* Diagnostic, no counterpart in the reference: compute units and peak engine clock (kHz) of the current device, the
- * two figures the SMFMAC peak is computed from (units x clock x 4096 dense fp16 FLOP per clock per unit x 2). */
-int onebit_sparse_device_info(int *compute_units, int *clock_khz);
 
 #ifdef __cplusplus
 }

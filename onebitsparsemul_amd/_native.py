@@ -6,8 +6,7 @@ import os
 import torch
 
 _DIR = os.path.dirname(os.path.abspath(__file__))
-# ONEBITMUL_LIBRARY overrides the in-tree build (e.g. to try an experimental build of the same ABI).
-LIB_PATH = os.environ.get("ONEBITMUL_LIBRARY") or os.path.join(_DIR, "libonebitmul.so")
+LIB_PATH = os.path.join(_DIR, "libonebitmul.so")
 
 F32, F16 = 0, 1
 META_REFERENCE, META_CUTLASS, META_LOGICAL = 0, 1, 2
@@ -17,6 +16,7 @@ EXPORTS = (
     "onebit_sparse_matmul_prepared", "onebit_sparse_matmul_prepared_static", "onebit_sparse_linear_prepared", "onebit_sparse_pack", "onebit_sparse_last_error", "onebit_sparse_set_tile_config",
     "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_set_split_k", "onebit_sparse_set_pad_b", "onebit_sparse_describe_launch", "onebit_sparse_set_weight_cache", "onebit_sparse_clear_weight_cache", "onebit_sparse_release_buffers",
     "onebit_sparse_measure_smfmac_rate", "onebit_sparse_device_info",
+    "onebit_sparse_describe_launch_for", "onebit_sparse_measure_smfmac_rate_shape",
 )
 
 _lib = None
@@ -65,6 +65,10 @@ def lib():
         L.onebit_sparse_release_buffers.argtypes = []
         L.onebit_sparse_describe_launch.restype = i32
         L.onebit_sparse_describe_launch.argtypes = [i32, i32, i32, i32, ctypes.POINTER(ctypes.c_int)]
+        L.onebit_sparse_describe_launch_for.restype = i32
+        L.onebit_sparse_describe_launch_for.argtypes = [i32, i32, i32, i32, i32, ctypes.POINTER(ctypes.c_int)]
+        L.onebit_sparse_measure_smfmac_rate_shape.restype = i32
+        L.onebit_sparse_measure_smfmac_rate_shape.argtypes = [i32, i32, i32, ctypes.POINTER(ctypes.c_double)]
         L.onebit_sparse_device_info.restype = i32
         L.onebit_sparse_device_info.argtypes = [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]
         L.onebit_sparse_measure_smfmac_rate.restype = i32
@@ -242,10 +246,13 @@ def set_pad_b(enabled):
     lib().onebit_sparse_set_pad_b(1 if enabled else 0)
 
 
-def measure_smfmac_rate(random_operands=True, iterations=50000):
-    """Sustained register-only SMFMAC rate of the current GPU, dense-equivalent TFLOP/s (diagnostic)."""
+SMFMAC_32X32X32, SMFMAC_16X16X64 = 0, 1
+
+
+def measure_smfmac_rate(random_operands=True, iterations=50000, shape=SMFMAC_32X32X32):
+    """Sustained register-only rate of one SMFMAC instruction on the current GPU, dense-equivalent TFLOP/s (diagnostic)."""
     out = ctypes.c_double(0.0)
-    rc = lib().onebit_sparse_measure_smfmac_rate(1 if random_operands else 0, iterations, ctypes.byref(out))
+    rc = lib().onebit_sparse_measure_smfmac_rate_shape(shape, 1 if random_operands else 0, iterations, ctypes.byref(out))
     if rc != 0:
         raise RuntimeError(f"libonebitmul: measuring the SMFMAC rate failed (status {rc})")
     return out.value
@@ -272,10 +279,14 @@ def device_info():
     return cus.value, khz.value
 
 
-def describe_launch(m, n, k, b_aligned=True):
-    """What a prepared call of this shape would launch (host-only): dict(kernel, rows or tile, splits, pad_b)."""
+def describe_launch(m, n, k, b_aligned=True, compute_units=256):
+    """What a prepared call of this shape would launch on a GPU with `compute_units` compute units (host-only; None = the
+    current device's count, which is what the calls themselves plan for): dict(kernel, rows or tile, splits, pad_b)."""
     plan = (ctypes.c_int * 4)()
-    _check(lib().onebit_sparse_describe_launch(m, n, k, 1 if b_aligned else 0, plan))
+    if compute_units is None:
+        _check(lib().onebit_sparse_describe_launch(m, n, k, 1 if b_aligned else 0, plan))
+    else:
+        _check(lib().onebit_sparse_describe_launch_for(m, n, k, 1 if b_aligned else 0, compute_units, plan))
     if plan[0]:
         return dict(kernel="skinny_kernel", rows=plan[1], splits=plan[2])
     return dict(kernel="gemm_kernel", tile=plan[1], splits=plan[2], pad_b=bool(plan[3]))

@@ -64,9 +64,22 @@ def build_binding():
     return out
 
 
+CONSUMER_SRC = os.path.join(ROOT, "tests", "consumer", "libso_test.cpp")
+CONSUMER_BIN = os.path.join(ROOT, "tests", "consumer", "libso_test")
+
+
+def build_consumer(out=CONSUMER_BIN):
+    """The C++ consumer of the boundary (the reference's `lib_test` target, makefile:22-23): declares the entry point
+    with C++ linkage as the reference's header does and links with -lonebitmul."""
+    _run([HIPCC, "-O1", "-std=c++17", CONSUMER_SRC, "-o", out, "-L", PKG, "-lonebitmul",
+          "-Wl,-rpath,$ORIGIN/../../onebitsparsemul_amd"])
+    return out
+
+
 def build_all():
     build_library()
     build_binding()
+    build_consumer()
 
 
 if __name__ == "__main__":

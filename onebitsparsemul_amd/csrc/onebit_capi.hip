@@ -1,7 +1,7 @@
 // C ABI of libonebitmul (declared in include/onebit_sparse_tensor.h): argument validation, per-device
 // workspaces, kernel selection. Host code only; the kernels live in onebit_kernels.hip.
 // Counterpart of the reference's host launcher csrc/kernel_lib.cu:23-97.
-#include "onebit_sparse_tensor.h"
+#include "onebit_sparse_tuning.h"
 #include "onebit_device.h"
 #include "onebit_launch.h"
 
@@ -442,16 +442,22 @@ void onebit_sparse_set_skinny_rows(int rows) { g_skinny_rows = rows; }
 void onebit_sparse_set_split_k(int splits) { g_split_k = splits; }
 void onebit_sparse_set_pad_b(int enabled) { g_pad_b = enabled ? 1 : 0; }
 
-int onebit_sparse_describe_launch(int m, int n, int k, int b_16_byte_aligned, int* plan) {
+int onebit_sparse_describe_launch_for(int m, int n, int k, int b_16_byte_aligned, int compute_units, int* plan) {
   g_last_error.clear();
   if (!plan) return fail(ONEBIT_ERR_ARGUMENT, "plan must not be null");
+  if (compute_units <= 0) return fail(ONEBIT_ERR_ARGUMENT, "compute_units must be positive (got %d)", compute_units);
   if (int rc = check_shape(m, n, k)) return rc;
-  const LaunchPlan p = choose_launch(m, n, k, b_16_byte_aligned != 0);
+  const LaunchPlan p = choose_launch(m, n, k, b_16_byte_aligned != 0, compute_units);
   plan[0] = p.split_k_kernel;
   plan[1] = p.rows_or_tile;
   plan[2] = p.splits;
   plan[3] = p.pad_b;
   return ONEBIT_OK;
+}
+
+int onebit_sparse_describe_launch(int m, int n, int k, int b_16_byte_aligned, int* plan) {
+  // the compute units of the current device, as the calls themselves plan; 256 when there is no usable device
+  return onebit_sparse_describe_launch_for(m, n, k, b_16_byte_aligned, current_compute_units(), plan);
 }
 
 size_t onebit_sparse_prepared_bytes(int m, int k) {

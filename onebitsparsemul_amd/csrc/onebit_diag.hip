@@ -2,7 +2,7 @@
 // memory inside the timed loop). The chip lowers its clock under matrix load, and by how much depends on the
 // operand values, so this is the practical ceiling the main kernel can be compared with next to the nominal peak.
 // No counterpart in the reference.
-#include "onebit_sparse_tensor.h"
+#include "onebit_sparse_tuning.h"
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -15,6 +15,7 @@ namespace {
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half16_t __attribute__((ext_vector_type(16)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef float float4v_t __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(256) void smfmac_rate_kernel(float* out, const half8_t* pa, const half16_t* pb,
                                                           const int* pidx, int iters) {
@@ -41,6 +42,32 @@ __global__ __launch_bounds__(256) void smfmac_rate_kernel(float* out, const half
   out[t] = s;
 }
 
+// The same loop on v_smfmac_f32_16x16x64_f16, the instruction of the default large tile and of the sixteen-column
+// split-K kernel: 16 independent 16 x 16 accumulator tiles per wavefront, 32768 dense-equivalent FLOPs per instruction.
+__global__ __launch_bounds__(256) void smfmac_rate_kernel_16x16x64(float* out, const half8_t* pa, const half16_t* pb,
+                                                                   const int* pidx, int iters) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  half8_t a[4];
+  half16_t b[4];
+  int idx[4];
+  for (int i = 0; i < 4; ++i) {
+    a[i] = pa[t * 4 + i];
+    b[i] = pb[t * 4 + i];
+    idx[i] = pidx[t * 4 + i];
+  }
+  float4v_t acc[16];
+  for (int j = 0; j < 16; ++j) acc[j] = float4v_t{0.f, 0.f, 0.f, 0.f};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      acc[j] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a[j & 3], b[(j >> 2) & 3], acc[j], idx[j & 3], 0, 0);
+  }
+  float s = 0.f;
+  for (int j = 0; j < 16; ++j)
+    for (int i = 0; i < 4; ++i) s += acc[j][i];
+  out[t] = s;
+}
+
 uint32_t lcg(uint32_t& state) {
   state = state * 1664525u + 1013904223u;
   return state >> 8;
@@ -48,8 +75,12 @@ uint32_t lcg(uint32_t& state) {
 
 }  // namespace
 
-extern "C" int onebit_sparse_measure_smfmac_rate(int random_operands, int iterations, double* dense_equiv_tflops) {
+extern "C" int onebit_sparse_measure_smfmac_rate_shape(int shape, int random_operands, int iterations,
+                                                       double* dense_equiv_tflops) {
   if (!dense_equiv_tflops || iterations <= 0) return ONEBIT_ERR_ARGUMENT;
+  if (shape != ONEBIT_SMFMAC_32X32X32 && shape != ONEBIT_SMFMAC_16X16X64) return ONEBIT_ERR_ARGUMENT;
+  auto kernel = shape == ONEBIT_SMFMAC_16X16X64 ? smfmac_rate_kernel_16x16x64 : smfmac_rate_kernel;
+  const double flops_per_instruction = shape == ONEBIT_SMFMAC_16X16X64 ? 2.0 * 16 * 16 * 64 : 2.0 * 32 * 32 * 32;
   int device = 0, cus = 0;
   if (hipGetDevice(&device) != hipSuccess) return ONEBIT_ERR_HIP;
   if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return ONEBIT_ERR_HIP;
@@ -84,14 +115,14 @@ extern "C" int onebit_sparse_measure_smfmac_rate(int random_operands, int iterat
   if (hipMemcpy(pb, hb.data(), hb.size() * 2, hipMemcpyHostToDevice) != hipSuccess) goto done;
   if (hipMemcpy(pidx, hi.data(), hi.size() * 4, hipMemcpyHostToDevice) != hipSuccess) goto done;
   if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) goto done;
-  hipLaunchKernelGGL(smfmac_rate_kernel, dim3(blocks), dim3(256), 0, nullptr, out, pa, pb, pidx, 200);
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, nullptr, out, pa, pb, pidx, 200);
   if (hipDeviceSynchronize() != hipSuccess) goto done;
   if (hipEventRecord(e0, nullptr) != hipSuccess) goto done;
-  hipLaunchKernelGGL(smfmac_rate_kernel, dim3(blocks), dim3(256), 0, nullptr, out, pa, pb, pidx, iterations);
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, nullptr, out, pa, pb, pidx, iterations);
   if (hipEventRecord(e1, nullptr) != hipSuccess) goto done;
   if (hipDeviceSynchronize() != hipSuccess) goto done;
   if (hipEventElapsedTime(&ms, e0, e1) != hipSuccess) goto done;
-  *dense_equiv_tflops = (double)blocks * 4 * iterations * 16 * 2.0 * 32 * 32 * 32 / (ms * 1e-3) / 1e12;
+  *dense_equiv_tflops = (double)blocks * 4 * iterations * 16 * flops_per_instruction / (ms * 1e-3) / 1e12;
   rc = ONEBIT_OK;
 done:
   // clean-up failures leave nothing to undo and do not change the measurement's outcome
@@ -102,6 +133,10 @@ done:
   (void)hipFree(pb);
   (void)hipFree(pidx);
   return rc;
+}
+
+extern "C" int onebit_sparse_measure_smfmac_rate(int random_operands, int iterations, double* dense_equiv_tflops) {
+  return onebit_sparse_measure_smfmac_rate_shape(ONEBIT_SMFMAC_32X32X32, random_operands, iterations, dense_equiv_tflops);
 }
 
 extern "C" int onebit_sparse_device_info(int* compute_units, int* clock_khz) {

@@ -1,5 +1,5 @@
 """The C ABI of libonebitmul.so as far as it can be exercised without a GPU: the library loads, exports every
-symbol that include/onebit_sparse_tensor.h declares, validates its arguments and reports HIP failures as
+symbol that include/onebit_sparse_tensor.h and include/onebit_sparse_tuning.h declare, validates its arguments and reports HIP failures as
 status codes (or, for the 8-argument symbol, as exit(EXIT_FAILURE) like the reference)."""
 import ctypes
 import os
@@ -12,14 +12,17 @@ import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "onebit_sparse_tensor.h")
+TUNING_HEADER = os.path.join(ROOT, "include", "onebit_sparse_tuning.h")
 
 from onebitsparsemul_amd import _native  # noqa: E402
 
 
-def _declared_functions():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(onebit_sparse_\w+)\s*\(", text)))
+def _declared_functions(*headers):
+    names = set()
+    for header in headers or (HEADER, TUNING_HEADER):
+        text = re.sub(r"/\*.*?\*/", "", open(header).read(), flags=re.S)
+        names |= set(re.findall(r"\b(onebit_sparse_\w+)\s*\(", text))
+    return sorted(names)
 
 
 def test_library_exports_every_declared_symbol():
@@ -33,8 +36,17 @@ def test_library_exports_every_declared_symbol():
     assert hasattr(lib, "_Z20onebit_sparse_matmulPvS_S_S_S_iii")
 
 
-def test_header_is_plain_c():
-    src = '#include "onebit_sparse_tensor.h"\nint main(void){return onebit_sparse_prepared_bytes(64,32)==0;}\n'
+def test_drop_in_header_holds_no_hooks_or_diagnostics():
+    """what a maintainer of the reference installs declares the product's entry points only"""
+    product = _declared_functions(HEADER)
+    assert not [n for n in product if "_set_tile" in n or "_set_skinny" in n or "_set_split" in n or "_set_pad" in n
+                or "describe" in n or "measure" in n or "device_info" in n]
+    assert "onebit_sparse_matmul" in product and "onebit_sparse_matmul_prepared_static" in product
+
+
+@pytest.mark.parametrize("header", ["onebit_sparse_tensor.h", "onebit_sparse_tuning.h"])
+def test_header_is_plain_c(header):
+    src = f'#include "{header}"\nint main(void){{return onebit_sparse_prepared_bytes(64,32)==0;}}\n'
     out = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-I", os.path.join(ROOT, "include"),
                           "-x", "c", "-"], input=src.encode(), capture_output=True)
     assert out.returncode == 0, out.stderr.decode()
@@ -190,6 +202,41 @@ def test_launch_plan_of_the_benchmark_shapes(_default_hooks):
     assert plan(4096, 1000, 4096, b_aligned=False)["pad_b"] is True
     assert plan(4096, 1000, 4096)["pad_b"] is False
     assert plan(256, 72, 128, b_aligned=False)["pad_b"] is False
+
+
+def test_hooks_act_on_the_calling_thread_only(_default_hooks):
+    """a hook set on one thread leaves the launches of every other thread alone"""
+    import threading
+    _native.set_skinny_enabled(False)
+    _native.set_tile_config(4)
+    seen = {}
+
+    def worker():
+        seen["plan"] = _native.describe_launch(11008, 16, 4096)
+        _native.set_skinny_rows(32)  # stays in the worker
+        seen["own"] = _native.describe_launch(28672, 16, 8192)
+
+    t = threading.Thread(target=worker)
+    t.start()
+    t.join()
+    assert seen["plan"] == dict(kernel="skinny_kernel", rows=64, splits=1)     # the defaults, not this thread's hooks
+    assert seen["own"] == dict(kernel="skinny_kernel", rows=32, splits=1)
+    assert _native.describe_launch(11008, 16, 4096)["kernel"] == "gemm_kernel"  # this thread's hooks still hold
+    _native.set_skinny_enabled(True)
+    _native.set_tile_config(-1)
+    assert _native.describe_launch(28672, 16, 8192) == dict(kernel="skinny_kernel", rows=128, splits=1)
+
+
+def test_launch_plan_scales_with_the_compute_units(_default_hooks):
+    """the explicit-count form plans for a smaller or partitioned GPU: fewer resident workgroups, other row groups"""
+    full = _native.describe_launch(28672, 16, 8192, compute_units=256)
+    small = _native.describe_launch(28672, 16, 8192, compute_units=64)
+    assert full == dict(kernel="skinny_kernel", rows=128, splits=1) and small["kernel"] == "skinny_kernel"
+    assert _native.describe_launch(2048, 16, 28672, compute_units=64)["splits"] <= 2   # one workgroup per compute unit
+    lib = _native.lib()
+    out = (ctypes.c_int * 4)()
+    assert lib.onebit_sparse_describe_launch_for(64, 8, 32, 1, 0, out) == 1
+    assert "compute_units" in _native.last_error()
 
 
 def test_launch_plan_follows_the_hooks(_default_hooks):

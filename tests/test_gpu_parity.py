@@ -544,6 +544,7 @@ def test_hip_graph_replays_match_eager(m, n, k):
     b = torch.zeros((k, n), dtype=torch.float16, device="cuda")
     d = torch.zeros((m, n), dtype=torch.float32, device="cuda")
     stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())  # prep, b and d were produced on the current stream
     with torch.cuda.stream(stream):
         _native.matmul_prepared(prep, b, d, m, n, k)  # eager warm-up on the capture stream
         stream.synchronize()

@@ -188,6 +188,7 @@ def test_linear_form_in_a_hip_graph(tokens, m, k):
     x = torch.zeros((tokens, k), dtype=torch.float16, device="cuda")
     y = torch.zeros((tokens, m), dtype=torch.float32, device="cuda")
     stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())  # prep, bias, x and y were produced on the current stream
     with torch.cuda.stream(stream):
         _native.linear_prepared(prep, x, y, m, k, bias=bias)
         stream.synchronize()

@@ -33,7 +33,7 @@ def test_two_calls_in_a_row_second_smaller():
     # (m, n, k): K split over workgroups and a padded copy of B in the first two, the split-K kernel with a K split over
     # workgroups in the third, a split of the main kernel alone in the fourth, no buffer at all in the last
     shapes = ((2048, 130, 8192), (1024, 100, 8192), (2048, 16, 16384), (512, 72, 4096), (1024, 16, 4096))
-    plans = [_native.describe_launch(m, n, k) for (m, n, k) in shapes]
+    plans = [_native.describe_launch(m, n, k, compute_units=None) for (m, n, k) in shapes]  # for this GPU
     assert plans[0]["splits"] > 1 and plans[0]["pad_b"] and plans[1]["splits"] > 1 and plans[1]["pad_b"]
     assert plans[2]["kernel"] == "skinny_kernel" and plans[2]["splits"] > 1   # the split-K kernel's own K split
     assert plans[3]["splits"] > 1 and plans[4] == dict(kernel="skinny_kernel", rows=32, splits=1)
@@ -66,3 +66,82 @@ def test_refuses_shapes_beyond_the_static_workspace():
         torch.cuda.synchronize()
     finally:
         _native.set_split_k(-1)
+
+
+def test_static_entry_point_is_capturable_without_a_warm_up():
+    """A call that allocated would invalidate the capture: the non-allocating entry point is captured in a HIP graph
+    with no eager call before it, on a shape that needs both internal buffers (K split over workgroups and a padded copy
+    of B), and every replay equals the eager result of the allocating entry point."""
+    for hook in (_native.set_tile_config, _native.set_skinny_rows, _native.set_split_k):
+        hook(-1)
+    m, n, k = 2048, 130, 8192
+    plan = _native.describe_launch(m, n, k, compute_units=None)
+    assert plan["splits"] > 1 and plan["pad_b"]
+    a, meta = synthetic.make_weight(m, k, seed=71)
+    prep = _native.prepare(a.cuda(), meta.cuda(), m, k)
+    b = torch.zeros((k, n), dtype=torch.float16, device="cuda")
+    d = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    # The entry point's first call on a device looks up the address of the static array (set-up, not an allocation);
+    # that happens here, outside the capture, through a shape that uses no internal buffer at all.
+    small = torch.zeros((64, 16), dtype=torch.float32, device="cuda")
+    _native.matmul_prepared(torch.zeros(_native.prepared_bytes(64, 256), dtype=torch.uint8, device="cuda"),
+                            torch.zeros((256, 16), dtype=torch.float16, device="cuda"), small, 64, 16, 256, static_scratch=True)
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            _native.matmul_prepared(prep, b, d, m, n, k, static_scratch=True)
+    for replay in range(3):
+        values = synthetic.make_b(k, n, seed=200 + replay, kind="int").cuda()
+        b.copy_(values)
+        d.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = torch.empty_like(d)
+        _native.matmul_prepared(prep, values, eager, m, n, k)
+        torch.cuda.synchronize()
+        assert torch.equal(d, eager) and bool(torch.isfinite(d).all())
+    ref = oracle.reference_matmul(a.numpy(), values.cpu().numpy(), meta.numpy(), m, n, k, d_dtype=oracle.F32)
+    assert np.array_equal(d.cpu().numpy(), ref)
+
+
+def test_allocating_entry_point_refuses_to_grow_under_capture_and_release_buffers():
+    """The allocating entry point cannot grow its buffers inside a capture: it refuses with a message, and the same call
+    works afterwards outside. onebit_sparse_release_buffers frees the buffers; the next split call allocates them again
+    and still matches the oracle."""
+    for hook in (_native.set_tile_config, _native.set_skinny_rows, _native.set_split_k):
+        hook(-1)
+    m, n, k = 1024, 72, 8192
+    assert _native.describe_launch(m, n, k, compute_units=None)["splits"] > 1
+    a, meta = synthetic.make_weight(m, k, seed=72)
+    bi = synthetic.make_b(k, n, seed=73, kind="int")
+    prep = _native.prepare(a.cuda(), meta.cuda(), m, k)
+    b = bi.cuda()
+    d = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    ref = oracle.reference_matmul(a.numpy(), bi.numpy(), meta.numpy(), m, n, k, d_dtype=oracle.F32)
+    torch.cuda.synchronize()
+    _native.release_buffers()  # whatever earlier tests left: this stream's K-split buffer has to be allocated anew
+    stream = torch.cuda.Stream()  # a fresh stream owns no library buffer yet
+    refused = None
+    with torch.cuda.stream(stream):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            try:
+                _native.matmul_prepared(prep, b, d, m, n, k)
+            except RuntimeError as err:
+                refused = str(err)
+    assert refused is not None and "being captured" in refused
+    del graph
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        _native.matmul_prepared(prep, b, d, m, n, k)  # the same call outside the capture allocates and runs
+    torch.cuda.synchronize()
+    assert np.array_equal(d.cpu().numpy(), ref)
+    _native.release_buffers()
+    d.fill_(float("nan"))
+    with torch.cuda.stream(stream):
+        _native.matmul_prepared(prep, b, d, m, n, k)  # allocates again after the release
+    torch.cuda.synchronize()
+    assert np.array_equal(d.cpu().numpy(), ref)
