@@ -528,17 +528,21 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
           _Pragma("unroll") for (int g = 0; g < 4 * FM; ++g)                                                        \
             if (g * FN / 4 == slot) AV[g / 4][g % 4] = expand_sign_register<(FILL_STEP)>(A_SRC[g / 4], one, g % 4);
 // the copies of stage S + 4 (and of the next chunk of A) behind SMFMAC `slot`: one by one when the stage is known to lie
-// inside K (A first, same request order), else all behind the first SMFMAC through the general, branching form
+// inside K (A first, same request order), else all behind the first SMFMAC through the general, branching form.
+// The copies are spread evenly over the region's slots: the wavefronts of a workgroup leave the barrier together, a
+// compute unit's address path takes one 16-byte-per-lane copy instruction per 16 clocks, and copies issued back to back
+// by every wavefront at once queue up there and hold the issuing wavefronts.
 #define ONEBIT_COPY_SLOT(S, ISSUE_A)                                                                               \
           if constexpr (FULL) {                                                                                    \
             constexpr int COPIES = ((ISSUE_A) ? NA : 0) + NL, CPS = (COPIES + SLOTS - 1) / SLOTS;                  \
+            constexpr int SPREAD = COPIES <= SLOTS ? SLOTS / COPIES : 1;  /* slots from one copy to the next */    \
             _Pragma("unroll") for (int c = 0; c < COPIES; ++c)                                                     \
-              if (c / CPS == slot) {                                                                               \
+              if ((c / CPS) * SPREAD == slot) {                                                                    \
                 const int i = c - ((ISSUE_A) ? NA : 0);                                                            \
                 if (i < 0) lds_dma16_base(a_chunk, a_off[c], a_dst[c]);                                            \
                 else lds_dma16_base(b_stage, b_off[i], lds_dst[i] + (S) * TS::STAGE_BYTES);                        \
               }                                                                                                    \
-            if (slot == (COPIES - 1) / CPS) {                                                                      \
+            if (slot == ((COPIES - 1) / CPS) * SPREAD) {                                                           \
               if (ISSUE_A) advance_a();                                                                            \
               b_stage += stage_stride;                                                                             \
               next_k0 += kStageK;                                                                                  \
@@ -579,18 +583,27 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
       struct ATile { uint32_t idx01, idx23, w01, w23; };
       const uint32_t half_select = (g16 >> 1) ? 0x07060302u : 0x05040100u;
       const int sign_shift = 4 * (g16 >> 1);
-      auto gather_a = [&](int rt) __attribute__((always_inline)) {
+      // A row tile's operands of one chunk in two steps, so that the LDS latency of the first lies under SMFMACs: the
+      // holder lane's 24 bytes as they are, then the selection of this lane's 16 index bits per stage and the shift
+      // of its sign words.
+      struct ARaw { u32x4_t meta; u32x2_t sign; };
+      auto load_a_raw = [&](int rt) __attribute__((always_inline)) {
         const char* block = a_frag_lds[rt >> 1];
         const int holder = c16 + 16 * (rt & 1) + 32 * (g16 & 1);
-        const u32x4_t meta = *reinterpret_cast<const u32x4_t*>(block + holder * 16);
-        const u32x2_t sign = *reinterpret_cast<const u32x2_t*>(block + kSignOffset + holder * 8);
+        ARaw r;
+        r.meta = *reinterpret_cast<const u32x4_t*>(block + holder * 16);
+        r.sign = *reinterpret_cast<const u32x2_t*>(block + kSignOffset + holder * 8);
+        return r;
+      };
+      auto finish_a = [&](const ARaw& r) __attribute__((always_inline)) {
         ATile t;
-        t.idx01 = __builtin_amdgcn_perm(meta.y, meta.x, half_select);
-        t.idx23 = __builtin_amdgcn_perm(meta.w, meta.z, half_select);
-        t.w01 = sign.x << sign_shift;
-        t.w23 = sign.y << sign_shift;
+        t.idx01 = __builtin_amdgcn_perm(r.meta.y, r.meta.x, half_select);
+        t.idx23 = __builtin_amdgcn_perm(r.meta.w, r.meta.z, half_select);
+        t.w01 = r.sign.x << sign_shift;
+        t.w23 = r.sign.y << sign_shift;
         return t;
       };
+      auto gather_a = [&](int rt) __attribute__((always_inline)) { return finish_a(load_a_raw(rt)); };
       // register p (kept values 2p, 2p+1) of the expanded signs of stage S
       auto expand16 = [&](const ATile& t, int S, int p_) __attribute__((always_inline)) {
         const uint32_t w = S < 2 ? t.w01 : t.w23;
@@ -651,10 +664,15 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
             }
           wait_vmcnt_lgkm0<WAITCNT>();  // copies of stage S+1 landed
           __builtin_amdgcn_s_barrier();
-          if constexpr (S == kStages - 1) {
-            // the next chunk of A is readable after this stage's barrier; row tiles 0-3 are done with this chunk
+          // Last stage of a chunk: the next chunk of A is readable after this stage's barrier. Row tiles 0-3 are done
+          // with this chunk: their holder lanes' bytes are requested right here and turned into operands behind the
+          // SMFMACs of column tile 1, by when they have arrived; row tiles 4-7 are multiplied to the end of the stage:
+          // requested behind column tile 5, turned into operands after the last SMFMAC.
+          constexpr bool LAST = S == kStages - 1;
+          ARaw a_raw[RT / 2];
+          if constexpr (LAST) {
 #pragma unroll
-            for (int rt = 0; rt < RT / 2; ++rt) a_cur[rt] = gather_a(rt);
+            for (int rt = 0; rt < RT / 2; ++rt) a_raw[rt] = load_a_raw(rt);
             __builtin_amdgcn_sched_barrier(0);
           }
           // second half: column tile by column tile against row tiles 4-7
@@ -668,15 +686,19 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
               ONEBIT_COPY_SLOT(S, ISSUE_A)
               // the fragment of column tile ct - 1 for the next stage, one read behind each of this tile's SMFMACs
               if (ct >= 1) read_b16((S + 1) % kStages, ct - 1, rl, bv);
+              if constexpr (LAST) {
+                if (ct == 1) a_cur[rl] = finish_a(a_raw[rl]);
+                if (ct == CT - 3) a_raw[rl] = load_a_raw(RT / 2 + rl);
+              }
               // signs of row tile 0 of the next stage
               if (ct == CT - 1) av_roll[0][rl] = expand16(a_cur[0], (S + 1) % kStages, rl);
               __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
           for (int q = 0; q < 4; ++q) read_b16((S + 1) % kStages, CT - 1, q, bv);
-          if constexpr (S == kStages - 1) {
+          if constexpr (LAST) {
 #pragma unroll
-            for (int rt = RT / 2; rt < RT; ++rt) a_cur[rt] = gather_a(rt);  // row tiles 4-7 are done with this chunk
+            for (int rl = 0; rl < RT / 2; ++rl) a_cur[RT / 2 + rl] = finish_a(a_raw[rl]);
           }
         };
         using std::integral_constant;
