@@ -324,7 +324,9 @@ def main():
         # the same kernel family where the weight is large enough for bandwidth, not latency, to set the time
         line["decode_n16_large"] = run_decode_rotating(28672, 8192, 16, launches=500)
         # the linear layer's token-major form of the same kernels (decode and prefill sized)
-        line["layer_form"] = [run_layer_form(11008, 4096, 16), run_layer_form(4096, 4096, 2048, launches=200)]
+        # (8192 tokens on an 8192 x 8192 weight: the token-major form of the 16x16x64 tile the headline figure runs on)
+        line["layer_form"] = [run_layer_form(11008, 4096, 16), run_layer_form(4096, 4096, 2048, launches=200),
+                              run_layer_form(8192, 8192, 8192, launches=40)]
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w, operands)
     print(json.dumps(line))

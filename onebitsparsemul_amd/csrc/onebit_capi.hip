@@ -549,13 +549,12 @@ int onebit_sparse_linear_prepared(const void* prepared, const void* x, const voi
     ONEBIT_HIP(onebit::launch_skinny_tokens(args, plan.rows_or_tile, static_cast<hipStream_t>(stream)));
     return ONEBIT_OK;
   }
-  // the linear layer's form has no 16x16x64 variant: the same tile on eight wavefronts
-  if (plan.rows_or_tile == onebit::kTile512x128m16) plan.rows_or_tile = onebit::kTile512x128w8;
   switch (plan.rows_or_tile) {
     case onebit::kTile256x128w: case onebit::kTile128x128s: case onebit::kTile512x128w8: case onebit::kTile256x128w8:
-    case onebit::kTile128x128w8: case onebit::kTile64x128: case onebit::kTile128x128k2: case onebit::kTile64x128k2: break;
+    case onebit::kTile128x128w8: case onebit::kTile64x128: case onebit::kTile128x128k2: case onebit::kTile64x128k2:
+    case onebit::kTile512x128m16: break;
     default:
-      return fail(ONEBIT_ERR_ARGUMENT, "tile configuration %d has no token-major variant (4, 6, 9 ... 14 have)",
+      return fail(ONEBIT_ERR_ARGUMENT, "tile configuration %d has no token-major variant (4, 6, 9 ... 15 have)",
                   plan.rows_or_tile);
   }
   if (onebit::prepared_bytes(m, k) >= (size_t(1) << 32))

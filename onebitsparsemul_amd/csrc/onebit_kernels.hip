@@ -330,7 +330,7 @@ __device__ __attribute__((aligned(16))) uint32_t g_zero16[4] = {0, 0, 0, 0};
 // p.m), the epilogue is y = acc + bias; a tile column is a token.
 template <int WM, int WN, int FM, int FN, bool DMA, bool TOKENS = false, int KG = 1, bool M16 = false>
 __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gemm_kernel(GemmArgs p) {
-  static_assert(!M16 || (DMA && !TOKENS && KG == 1 && WN == 1 && FM == 4 && FN == 4), "the 16x16x64 form exists for the 512x128 four-wavefront tile");
+  static_assert(!M16 || (DMA && KG == 1 && WN == 1 && FM == 4 && FN == 4), "the 16x16x64 form exists for the 512x128 four-wavefront tile");
   static_assert(DMA || !TOKENS, "the token-major form uses the asynchronous copies");
   static_assert(DMA || KG == 1, "the two-group form uses the asynchronous copies");
   using TS = TileShape<WM, WN, FM, FN, KG>;
@@ -573,7 +573,18 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct)
         ct_off[ct] = (((2 * (wn * CT + ct) + ((c16 & 3) >> 1)) ^ chunk_swizzle<BN>(brow)) << 4) + (c16 & 1) * 8;
+      // Token-major image (linear-layer form): the operand of token 16 ct + c16 is pieces g16 and 4 + g16 of its row, two plain
+      // 16-byte reads (q = 0, 1); the swizzle of a token row depends on c16 alone, so the column tile is an immediate offset.
+      const int token_piece = c16 * (kStageK * 2) + ((g16 ^ token_swizzle(c16)) << 4);
       auto read_b16 = [&](int ring_slot, int ct, int q, u32x8_t* bv) __attribute__((always_inline)) {
+        if constexpr (TOKENS) {
+          if (q < 2) {
+            const u32x4_t t = *reinterpret_cast<const u32x4_t*>(smem + ring_slot * TS::STAGE_BYTES + ct * (16 * kStageK * 2) +
+                                                                 (token_piece ^ (q << 6)));
+            bv[ct][4 * q] = t.x; bv[ct][4 * q + 1] = t.y; bv[ct][4 * q + 2] = t.z; bv[ct][4 * q + 3] = t.w;
+          }
+          return;
+        }
         const int row_const = 4 * (q & 1) + 32 * (q >> 1);
         const u32x2_t t = lds_read_tr16(smem + ring_slot * TS::STAGE_BYTES + brow_off + row_const * (BN * 2) + ct_off[ct]);
         bv[ct][2 * q] = t.x;
@@ -944,12 +955,26 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
 #pragma unroll
       for (int fm = 0; fm < FM; ++fm) {
         if (!finishes(fm)) continue;  // the other K group stores this fragment
+        if constexpr (M16) {
+          // 16x16x64 form: the four registers of tile (2 fm + rh, ct) are rows 16 rh + 4 (lane / 16) ... + 3 of token
+          // 16 ct + lane % 16: slot 4 rh + lane / 16 of that token's line
+          const int g16 = lane >> 4, c16 = lane & 15;
+#pragma unroll
+          for (int rh = 0; rh < 2; ++rh)
+#pragma unroll
+            for (int ct = 0; ct < 2 * FN; ++ct) {
+              const float4v_t v4 = acc16[2 * fm + rh][ct];
+              *reinterpret_cast<float4*>(scratch + (ct * 16 + c16) * 128 + (((4 * rh + g16) ^ token_swizzle(c16)) << 4)) =
+                  float4{v4[0], v4[1], v4[2], v4[3]};
+            }
+        } else {
 #pragma unroll
         for (int fn = 0; fn < FN; ++fn)
 #pragma unroll
           for (int q = 0; q < 4; ++q)
             *reinterpret_cast<float4*>(scratch + (fn * 32 + token_lane) * 128 + (((2 * q + gb) ^ token_swizzle(token_lane)) << 4)) =
                 float4{acc[fm][fn][4 * q], acc[fm][fn][4 * q + 1], acc[fm][fn][4 * q + 2], acc[fm][fn][4 * q + 3]};
+        }
         const int row_base = row0 + fm * 32;
         if (p.d_f16) {
 #pragma unroll
@@ -988,6 +1013,23 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
       return;
     }
     // y not 16-byte aligned: one element per accumulator register
+    if constexpr (M16) {
+#pragma unroll
+      for (int rt = 0; rt < 2 * FM; ++rt)
+#pragma unroll
+        for (int ct = 0; ct < 2 * FN; ++ct)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int token = col0 + ct * 16 + (lane & 15), row = row0 + rt * 16 + 4 * (lane >> 4) + v;
+            if (token < p.n && row < row_limit) {
+              const float x = acc16[rt][ct][v] + bias_of(row);
+              const size_t o = (size_t)token * p.m + row;
+              if (p.d_f16) reinterpret_cast<_Float16*>(d_out)[o] = (_Float16)x;
+              else reinterpret_cast<float*>(d_out)[o] = x;
+            }
+          }
+      return;
+    }
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm) {
       if (!finishes(fm)) continue;  // the other K group stores this fragment
@@ -2029,6 +2071,7 @@ hipError_t launch_gemm_tokens(GemmArgs args, int tile_config, hipStream_t stream
       case kTile64x128: return launch_gemm_cfg<2, 2, 1, 2, true, true>(a, stream);
       case kTile128x128k2: return launch_gemm_cfg<2, 2, 2, 2, true, true, 2>(a, stream);
       case kTile64x128k2: return launch_gemm_cfg<2, 2, 1, 2, true, true, 2>(a, stream);
+      case kTile512x128m16: return launch_gemm_cfg<4, 1, 4, 4, true, true, 1, true>(a, stream);
       default: return hipErrorInvalidValue;  // the tiles the automatic choice uses
     }
   };

@@ -60,7 +60,7 @@ hipError_t launch_prepare(const void* a, const void* e, void* prep, int m, int k
 hipError_t launch_gemm(GemmArgs args, int tile_config, hipStream_t stream);
 // The linear layer's form of the main kernel: b is x (n tokens x k, token-major, 16-byte aligned), d is y (n tokens x
 // m), y = x W^T + bias; c, alpha, beta and the padded copy of B are not used, splits / chunks_per_split / split_ws as in
-// launch_gemm. Tiles 4, 6, 9, 10, 11, 12, 13, 14.
+// launch_gemm. Tiles 4, 6, 9, 10, 11, 12, 13, 14, 15.
 hipError_t launch_gemm_tokens(GemmArgs args, int tile_config, hipStream_t stream);
 // dense fp16 (m x k) -> one-bit values `a` and metadata `e`; prune != 0 applies the 2:4 magnitude mask first
 hipError_t launch_pack(const void* w, void* a, void* e, int m, int k, int prune, int layout, hipStream_t stream);

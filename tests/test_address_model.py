@@ -441,7 +441,7 @@ def test_every_tile_configuration(hooks, tile):
     _native.set_skinny_enabled(False)
     for m, n, k in ((1024, 512, 1024), (576, 264, 192), (2112, 1032, 64), (8192, 8192, 8192)):
         check_call(m, n, k)
-        if tile in (4, 6, 9, 10, 11, 12, 13, 14):
+        if tile in (4, 6, 9, 10, 11, 12, 13, 14, 15):
             check_call(m, n, k, tokens=True)
 
 

@@ -49,7 +49,7 @@ def test_linear_form_small_token_counts(rows, tokens, m, k):
         assert np.array_equal(y.cpu().numpy(), want), (y_dtype, b is not None)
 
 
-@pytest.mark.parametrize("tile", [-1, 4, 6, 9, 10, 11, 12, 13, 14])
+@pytest.mark.parametrize("tile", [-1, 4, 6, 9, 10, 11, 12, 13, 14, 15])
 @pytest.mark.parametrize("tokens,m,k", [(65, 256, 512), (128, 192, 1056), (200, 1024, 2048), (1000, 640, 544), (16, 256, 800),
                                         (520, 4096, 512)])
 def test_linear_form_main_kernel(tile, tokens, m, k):

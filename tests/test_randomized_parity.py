@@ -64,7 +64,7 @@ def test_random_cases_match_the_oracle(seed):
         torch.cuda.synchronize()
         assert np.array_equal(d.cpu().numpy(), want), what
         # the layer's form of the same product (tiles without a token-major variant: automatic choice)
-        if hooks["tile"] not in (-1, 4, 6, 9, 10, 11, 12, 13, 14):
+        if hooks["tile"] not in (-1, 4, 6, 9, 10, 11, 12, 13, 14, 15):
             _native.set_tile_config(-1)
         plain = oracle.host_gemm(dense, bi.numpy(), d_dtype=oracle.F32, acc="f32")
         bias = synthetic.make_b(1, m, seed=case + 2, kind="int").reshape(m)
