@@ -133,6 +133,27 @@ def run_decode_rotating(m, k, n, launches=2000, copies=None):
                 frac_of_hbm_peak=nbytes / t_rot / 1e9 / HBM_PEAK_GBS)
 
 
+def run_decode_grouped(m, k, tokens, group=8, launches=400):
+    """The grouped entry point on decode-sized products: `group` distinct weights of m x k per launch (one launch of the
+    split-K kernel for all of them), rotating over enough sets that every launch streams its weights from HBM; next to
+    the single-launch figure, never instead of it. Token-major x and y as the layer holds them."""
+    import torch
+    from onebitsparsemul_amd import _native, synthetic
+    a, meta = synthetic.make_weight(m, k, seed=3, device="cuda")
+    prep0 = _native.prepare(a, meta, m, k)
+    sets = max(4, (768 << 20) // (prep0.numel() * group) + 1)
+    x = synthetic.make_b(tokens, k, seed=4, kind="normal", device="cuda")
+    problems = []
+    for s_ in range(sets):
+        problems.append([(prep0 if s_ + g == 0 else prep0.clone(), x, torch.empty((tokens, m), dtype=torch.float16, device="cuda"),
+                          m, k, None) for g in range(group)])
+    t = time_graph(lambda i: _native.linear_prepared_grouped(problems[i % sets]), launches)
+    nbytes = algorithmic_bytes(m, tokens, k, 0.0)
+    return dict(shape=f"{group} x ({m}x{k}, {tokens} tokens) per launch", bytes_per_problem=nbytes, sets=sets, launches=launches,
+                us_per_launch=t * 1e6, us_per_problem=t * 1e6 / group, gbps_hbm=nbytes * group / t / 1e9,
+                frac_of_hbm_peak=nbytes * group / t / 1e9 / HBM_PEAK_GBS)
+
+
 def run_layer_form(m, k, tokens, launches=1000):
     """The linear layer's call y = x W^T + bias (x and y token-major) three ways, each inside a HIP graph: the
     token-major kernel form, the plain kernel on operands that are already transposed (no bias), and the plain kernel
@@ -323,6 +344,8 @@ def main():
         line["decode_n16"] = run_decode_rotating(11008, 4096, 16)
         # the same kernel family where the weight is large enough for bandwidth, not latency, to set the time
         line["decode_n16_large"] = run_decode_rotating(28672, 8192, 16, launches=500)
+        # several decode-sized products in one launch (the grouped entry point): 8 distinct weights per launch
+        line["decode_n16_grouped"] = run_decode_grouped(11008, 4096, 16)
         # the linear layer's token-major form of the same kernels (decode and prefill sized)
         # (8192 tokens on an 8192 x 8192 weight: the token-major form of the 16x16x64 tile the headline figure runs on)
         line["layer_form"] = [run_layer_form(11008, 4096, 16), run_layer_form(4096, 4096, 2048, launches=200),

@@ -109,6 +109,29 @@ int onebit_sparse_linear_prepared(const void *prepared, const void *x, const voi
                                   int k, int bias_dtype, int y_dtype, void *stream);
 
 /*
+ * Grouped linear-layer form: `count` independent products y_i = x_i W_i^T (+ bias_i) that share the token count, each
+ * with its own prepared weight (m_i x k_i), activations x_i (tokens x k_i), bias_i (m_i values or NULL) and result y_i
+ * (tokens x m_i); the x_i may be one and the same buffer. `problems` is a HOST array, read before the call returns.
+ * For the callers of BinaryLinear_2_4.forward that issue several projections of one layer back to back (q / k / v,
+ * gate / up: onebit_sparse_mul/__init__.py:118-128 called once per projection): with tokens <= 64 every 16 problems are
+ * one launch of the split-K kernel, whose workgroups are numbered over the concatenated row groups of the problems, so
+ * that the launch and the start of the memory stream are paid once instead of per projection (decode-sized products
+ * take a few microseconds each, half of which is that). Results are identical to `count` calls of
+ * onebit_sparse_linear_prepared without a K split over workgroups (same sums in the same order per element). With
+ * tokens > 64 it is exactly such a sequence of calls. bias_dtype and y_dtype hold for all problems. No counterpart in
+ * the reference (one launch per product, csrc/kernel_lib.cu:86); allocates nothing.
+ */
+typedef struct onebit_linear_problem {
+  const void *prepared; /* from onebit_sparse_prepare, m x k */
+  const void *x;        /* fp16, tokens x k, row-major, 16-byte aligned */
+  const void *bias;     /* m values (bias_dtype) or NULL */
+  void *y;              /* tokens x m, row-major (y_dtype) */
+  int m, k;
+} onebit_linear_problem;
+int onebit_sparse_linear_prepared_grouped(const onebit_linear_problem *problems, int count, int tokens, int bias_dtype,
+                                          int y_dtype, void *stream);
+
+/*
  * Packs a dense fp16 weight (m x k, row-major, device) into the stored operands a (m*k/16 bytes) and e
  * (m*k/8 bytes) on the GPU. Replaces the tensor-op pipeline of BinaryLinear_2_4.pack
  * (onebit_sparse_mul/__init__.py:130-145 with _semi_structured_conversions.py:54-179,286-314): prune != 0 first

@@ -202,3 +202,47 @@ class BinaryLinear_2_4(nn.Module):
         y = self._prepared.linear(tokens, bias=bias.contiguous() if bias is not None else None, out_dtype=out_dtype)
         y = y.reshape(*lead, self.outfeatures)
         return y if self.out_dtype is not None else y.to(x.dtype)
+
+
+def forward_grouped(layers, xs):
+    """The forward passes of several BinaryLinear_2_4 layers on inputs with the same number of tokens, in one library
+    call (one kernel launch per 16 layers for up to 64 tokens): the q / k / v or gate / up projections of a decoder
+    layer. xs: one tensor for all layers, or one per layer. Returns the list of outputs, each what layer(x) returns."""
+    if isinstance(xs, torch.Tensor):
+        xs = [xs] * len(layers)
+    if len(xs) != len(layers):
+        raise ValueError("one input per layer (or one for all)")
+    if not layers:
+        return []
+    flat, prepared = {}, []
+    for layer, x in zip(layers, xs):
+        if not layer.vaild:
+            raise NotImplementedError("a BinaryLinear_2_4 layer holds no packed weight: call pack() first")
+        if layer._prepared is None or layer._prepared.buffer.device != x.device:
+            layer._prepared = PreparedWeight(layer.packed_binary_sparse.to(x.device), layer.meta.to(x.device))
+        if id(x) not in flat:  # inputs shared by several layers are made contiguous fp16 once
+            t = x.reshape(-1, layer.infeatures).to(torch.float16).contiguous()
+            flat[id(x)] = t.clone() if t.data_ptr() % 16 else t
+        prepared.append(flat[id(x)])
+    tokens = prepared[0].shape[0]
+    out_dtypes = {layer.out_dtype or (torch.float16 if x.dtype == torch.float16 else torch.float32)
+                  for layer, x in zip(layers, xs)}
+    bias_dtypes = {layer.bias.dtype if layer.bias.dtype in (torch.float16, torch.float32) else torch.float32
+                   for layer in layers if layer.bias is not None}
+    if tokens == 0 or len(out_dtypes) > 1 or len(bias_dtypes) > 1 or any(t.shape[0] != tokens for t in prepared):
+        return [layer(x) for layer, x in zip(layers, xs)]  # nothing to share: the layers one by one
+    out_dtype = out_dtypes.pop()
+    problems, ys = [], []
+    for layer, x, t in zip(layers, xs, prepared):
+        bias = layer.bias
+        if bias is not None:
+            bias = bias.to(device=x.device, dtype=bias_dtypes and next(iter(bias_dtypes))).contiguous()
+        y = torch.empty((tokens, layer.outfeatures), dtype=out_dtype, device=x.device)
+        problems.append((layer._prepared.buffer, t, y, layer.outfeatures, layer.infeatures, bias))
+        ys.append(y)
+    _native.linear_prepared_grouped(problems)
+    outs = []
+    for layer, x, y in zip(layers, xs, ys):
+        y = y.reshape(*x.shape[:-1], layer.outfeatures)
+        outs.append(y if layer.out_dtype is not None else y.to(x.dtype))
+    return outs

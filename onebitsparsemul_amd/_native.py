@@ -17,7 +17,14 @@ EXPORTS = (
     "onebit_sparse_set_skinny_enabled", "onebit_sparse_set_skinny_rows", "onebit_sparse_set_split_k", "onebit_sparse_set_pad_b", "onebit_sparse_describe_launch", "onebit_sparse_set_weight_cache", "onebit_sparse_clear_weight_cache", "onebit_sparse_release_buffers",
     "onebit_sparse_measure_smfmac_rate", "onebit_sparse_device_info",
     "onebit_sparse_describe_launch_for", "onebit_sparse_measure_smfmac_rate_shape",
+    "onebit_sparse_linear_prepared_grouped",
 )
+
+
+class LinearProblem(ctypes.Structure):
+    """onebit_linear_problem of include/onebit_sparse_tensor.h"""
+    _fields_ = [("prepared", ctypes.c_void_p), ("x", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("y", ctypes.c_void_p),
+                ("m", ctypes.c_int), ("k", ctypes.c_int)]
 
 _lib = None
 
@@ -43,6 +50,8 @@ def lib():
         L.onebit_sparse_matmul_prepared_static.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, i32, vp]
         L.onebit_sparse_linear_prepared.restype = i32
         L.onebit_sparse_linear_prepared.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp]
+        L.onebit_sparse_linear_prepared_grouped.restype = i32
+        L.onebit_sparse_linear_prepared_grouped.argtypes = [ctypes.POINTER(LinearProblem), i32, i32, i32, i32, vp]
         L.onebit_sparse_pack.restype = i32
         L.onebit_sparse_pack.argtypes = [vp, i32, i32, i32, vp, vp, i32, vp]
         L.onebit_sparse_last_error.restype = ctypes.c_char_p
@@ -187,6 +196,38 @@ def linear_prepared(prepared, x, y, m, k, bias=None):
             prepared.data_ptr(), x.data_ptr(), bias.data_ptr() if bias is not None else None, y.data_ptr(), tokens, m, k,
             _dtype_code(bias) if bias is not None else F16, _dtype_code(y), _stream(x)))
     return y
+
+
+def linear_prepared_grouped(problems):
+    """Several products y_i = x_i @ W_i.T (+ bias_i) with the same token count in one call (one launch per 16 problems
+    when tokens <= 64). problems: sequence of (prepared, x, y, m, k, bias or None); all y of one dtype, all biases of one."""
+    if not problems:
+        return
+    tokens = problems[0][1].shape[0]
+    table = (LinearProblem * len(problems))()
+    dev = None
+    bias_code, y_code = F16, None
+    for i, (prepared, x, y, m, k, bias) in enumerate(problems):
+        dev = _require_cuda(prepared, x, y, bias)
+        if x.dtype != torch.float16 or tuple(x.shape) != (tokens, k):
+            raise ValueError("every x must be float16 of shape (tokens, k) with the same token count")
+        if tuple(y.shape) != (tokens, m) or (bias is not None and tuple(bias.shape) != (m,)):
+            raise ValueError("y must have shape (tokens, m) and bias (m,)")
+        if prepared.numel() != _prepared_bytes_fast(m, k):
+            raise ValueError("prepared operand does not match m, k")
+        if y_code is not None and _dtype_code(y) != y_code:
+            raise TypeError("all results must have the same dtype")
+        y_code = _dtype_code(y)
+        if bias is not None:
+            code = _dtype_code(bias)
+            if any(p[5] is not None and _dtype_code(p[5]) != code for p in problems[:i]):
+                raise TypeError("all biases must have the same dtype")
+            bias_code = code
+        table[i] = LinearProblem(prepared.data_ptr(), x.data_ptr(), bias.data_ptr() if bias is not None else None,
+                                 y.data_ptr(), m, k)
+    with _on_device(dev):
+        _check(lib().onebit_sparse_linear_prepared_grouped(table, len(problems), tokens, bias_code, y_code,
+                                                           _stream(problems[0][1])))
 
 
 def _check_stored_operands(a, meta, c, d, m, n, k):

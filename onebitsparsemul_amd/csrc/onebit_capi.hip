@@ -590,6 +590,61 @@ int onebit_sparse_linear_prepared(const void* prepared, const void* x, const voi
   return ONEBIT_OK;
 }
 
+int onebit_sparse_linear_prepared_grouped(const onebit_linear_problem* problems, int count, int tokens, int bias_dtype,
+                                          int y_dtype, void* stream) {
+  g_last_error.clear();
+  if (!problems || count < 1) return fail(ONEBIT_ERR_ARGUMENT, "problems must point to at least one problem (count = %d)", count);
+  if (int rc = check_dtype(bias_dtype, y_dtype)) return rc;
+  for (int i = 0; i < count; ++i) {
+    const onebit_linear_problem& q = problems[i];
+    if (int rc = check_shape(q.m, tokens, q.k)) return rc;
+    if (!q.prepared || !q.x || !q.y) return fail(ONEBIT_ERR_ARGUMENT, "null operand pointer in problem %d", i);
+    if ((reinterpret_cast<uintptr_t>(q.x) & 15) != 0) return fail(ONEBIT_ERR_ARGUMENT, "x of problem %d must be 16-byte aligned", i);
+    if ((size_t)q.k * 256 * 2 >= (size_t(1) << 32))
+      return fail(ONEBIT_ERR_ARGUMENT, "the token-major form addresses x with 32-bit offsets inside a tile of 256 tokens: "
+                                       "k = %d of problem %d is beyond its limit of 8388607", q.k, i);
+  }
+  // Beyond the split-K kernel's range of token counts, or with that kernel switched off, there is nothing to share:
+  // one call of the single form per problem.
+  if (tokens > onebit::kSkinnyMaxN || !g_skinny_enabled) {
+    for (int i = 0; i < count; ++i) {
+      const onebit_linear_problem& q = problems[i];
+      if (int rc = onebit_sparse_linear_prepared(q.prepared, q.x, q.bias, q.y, tokens, q.m, q.k, bias_dtype, y_dtype, stream))
+        return rc;
+    }
+    return ONEBIT_OK;
+  }
+  // Row group of the launch: as for one product with all the weight rows, the largest that still gives about two
+  // workgroups per three compute units.
+  const int compute_units = current_compute_units();
+  for (int first = 0; first < count; first += onebit::kSkinnyMaxGroup) {
+    const int in_launch = std::min(count - first, onebit::kSkinnyMaxGroup);
+    long rows_total = 0;
+    for (int i = 0; i < in_launch; ++i) rows_total += problems[first + i].m;
+    const int enough = std::max(1, 160 * compute_units / 256);
+    const int rows = g_skinny_rows > 0 ? g_skinny_rows
+                     : (rows_total / 128 >= enough && tokens <= 32) ? 128 : (rows_total / 64 >= enough) ? 64 : 32;
+    if (rows != 32 && rows != 64 && rows != 128) return fail(ONEBIT_ERR_ARGUMENT, "row group %d: must be 32, 64 or 128", rows);
+    onebit::SkinnyGroupArgs group{};
+    group.count = in_launch;
+    for (int i = 0; i < in_launch; ++i) {
+      const onebit_linear_problem& q = problems[first + i];
+      onebit::SkinnyArgs& args = group.problem[i];
+      args.prep = static_cast<const uint8_t*>(q.prepared);
+      args.b = static_cast<const _Float16*>(q.x);
+      args.d = q.y;
+      args.m = q.m; args.n = tokens; args.k = q.k;
+      args.kc_total = (q.k + onebit::kChunkK - 1) / onebit::kChunkK;
+      args.alpha = 1.f; args.beta = 0.f;
+      args.d_f16 = y_dtype == ONEBIT_DTYPE_F16;
+      args.bias = q.bias;
+      args.bias_f16 = bias_dtype == ONEBIT_DTYPE_F16;
+    }
+    ONEBIT_HIP(onebit::launch_skinny_group(group, rows, static_cast<hipStream_t>(stream)));
+  }
+  return ONEBIT_OK;
+}
+
 int onebit_sparse_matmul_ex(const void* a, const void* b, const void* c, void* d, const void* e, int m, int n, int k,
                             float alpha, float beta, int c_dtype, int d_dtype, int meta_layout, void* stream) {
   g_last_error.clear();

@@ -1370,8 +1370,9 @@ __device__ __forceinline__ u32x4_t skinny_load_piece(const _Float16* __restrict_
   return v;
 }
 
+// The body of the split-K kernel for workgroup (block_x, block_y) of problem p: block_x = row group, block_y = K split.
 template <int NW, int R, int MODE, int NC>
-__global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(SkinnyArgs p) {
+__device__ __forceinline__ void skinny_body(const SkinnyArgs& p, const int block_x, const int block_y) {
   constexpr int NT = 64 * NW;
   constexpr int IMG_ROWS = kSkinnyRegion / (NC * 2);   // B rows per image: 256, 128 or 64
   constexpr int SUB = kChunkK / IMG_ROWS;              // images per chunk: 1, 2 or 4
@@ -1396,7 +1397,7 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int rb_total = p.m / kRowBlock;
-  const int rb_first = blockIdx.x * R;
+  const int rb_first = block_x * R;
   char* region = bs + wave * kSkinnyRegion;
   // kernel arguments the lambdas use, as values (capturing the argument struct would move it to scratch memory)
   const _Float16* __restrict__ b_ptr = p.b;
@@ -1425,7 +1426,7 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
   };
   // K split over workgroups (grid.y > 1): this workgroup multiplies the chunks [kc_begin, kc_end) and writes raw fp32
   // sums to its slice of the partial-sum buffer; a second kernel adds the slices in order and applies the epilogue.
-  const int kc_begin = blockIdx.y * p.chunks_per_split;
+  const int kc_begin = block_y * p.chunks_per_split;
   const int kc_end = kc_begin + p.chunks_per_split < kc_total ? kc_begin + p.chunks_per_split : kc_total;
   const int first = kc_begin + wave;  // this wavefront's first chunk
   // Short K (at most two chunks per wavefront, e.g. 11008 x 4096): everything the wavefront will read is requested
@@ -1765,7 +1766,7 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
     for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4_t*>(region + (lane + i * 64) * 16) = u32x4_t{0, 0, 0, 0};
   }
   u32x4_t breg[8];
-  char* const d_out = reinterpret_cast<char*>(p.d) + (size_t)blockIdx.y * p.m * p.n * (p.d_f16 ? 2 : 4);
+  char* const d_out = reinterpret_cast<char*>(p.d) + (size_t)block_y * p.m * p.n * (p.d_f16 ? 2 : 4);
   if (short_k) {
     u32x4_t breg2[8];
     load_b(first * kChunkK, breg);
@@ -1894,6 +1895,25 @@ __global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(Skinn
       }
     }
   }
+}
+
+template <int NW, int R, int MODE, int NC>
+__global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_kernel(SkinnyArgs p) {
+  skinny_body<NW, R, MODE, NC>(p, blockIdx.x, blockIdx.y);
+}
+
+// Grouped form: several independent products y_i = x_i W_i^T + bias_i that share the token count, in one launch. The
+// workgroups are numbered over the concatenated row groups of the problems; a workgroup finds its problem by
+// comparing its number with the problems' first workgroups (wave-uniform, a handful of scalar compares) and then runs
+// the token-major body on that problem's arguments. Decode-sized products take a few microseconds each, of which the
+// launch itself and the ramp of the memory pipeline are a large part: one launch for the q / k / v or gate / up
+// projections of a layer pays them once.
+template <int NW, int R, int NC>
+__global__ __launch_bounds__(64 * NW, NW == 16 ? 4 : 2) void skinny_group_kernel(SkinnyGroupArgs g) {
+  int which = 0;
+  for (int i = 1; i < g.count; ++i)
+    if ((int)blockIdx.x >= g.first_block[i]) which = i;
+  skinny_body<NW, R, kSkinnyBTokens, NC>(g.problem[which], (int)blockIdx.x - g.first_block[which], 0);
 }
 
 // =====================================================================================================
@@ -2202,6 +2222,40 @@ hipError_t launch_skinny_tokens(SkinnyArgs args, int rows_per_group, hipStream_t
   if (st != hipSuccess || args.splits <= 1) return st;
   return launch_split_reduce(args.split_ws, args.splits, (size_t)args.m * args.n, nullptr, args.d, 1.f, 0.f, 0, args.d_f16,
                              args.bias, args.bias_f16, args.m, stream);
+}
+
+template <int NW, int R>
+static hipError_t launch_skinny_group_cfg(const SkinnyGroupArgs& g, int blocks, int tokens, hipStream_t stream) {
+  if (tokens > 32) hipLaunchKernelGGL((skinny_group_kernel<NW, (R > 2 ? 2 : R), 64>), dim3(blocks), dim3(64 * NW), 0, stream, g);
+  else if (tokens > 16) hipLaunchKernelGGL((skinny_group_kernel<NW, R, 32>), dim3(blocks), dim3(64 * NW), 0, stream, g);
+  else hipLaunchKernelGGL((skinny_group_kernel<NW, R, 16>), dim3(blocks), dim3(64 * NW), 0, stream, g);
+  return hipGetLastError();
+}
+
+hipError_t launch_skinny_group(SkinnyGroupArgs g, int rows_per_group, hipStream_t stream) {
+  if (g.count < 1 || g.count > kSkinnyMaxGroup) return hipErrorInvalidValue;
+  const int tokens = g.problem[0].n;
+  if (tokens < 1 || tokens > kSkinnyMaxN) return hipErrorInvalidValue;
+  if (rows_per_group != 32 && rows_per_group != 64 && rows_per_group != 128) return hipErrorInvalidValue;
+  const int rows = (rows_per_group == 128 && tokens > 32) ? 64 : rows_per_group;  // as launch_skinny_tokens_cfg does
+  int blocks = 0;
+  for (int i = 0; i < g.count; ++i) {
+    SkinnyArgs& p = g.problem[i];
+    if (p.n != tokens || p.m <= 0 || p.k <= 0 || !p.prep || !p.b || !p.d) return hipErrorInvalidValue;
+    // 16-byte loads of x; lane offsets of up to 64 token rows must stay below the "outside" offset of the kernel
+    if ((reinterpret_cast<uintptr_t>(p.b) & 15) != 0 || (size_t)p.k * 64 * 2 >= 0xFFFFFF00u) return hipErrorInvalidValue;
+    p.splits = 1;
+    p.chunks_per_split = p.kc_total;
+    p.split_ws = nullptr;
+    g.first_block[i] = blocks;
+    blocks += (p.m + rows - 1) / rows;
+  }
+  g.first_block[g.count] = blocks;
+  switch (rows_per_group) {
+    case 32: return launch_skinny_group_cfg<16, 1>(g, blocks, tokens, stream);
+    case 64: return launch_skinny_group_cfg<8, 2>(g, blocks, tokens, stream);
+    default: return launch_skinny_group_cfg<8, 4>(g, blocks, tokens, stream);
+  }
 }
 
 hipError_t launch_skinny(SkinnyArgs args, int rows_per_group, hipStream_t stream) {

@@ -54,6 +54,15 @@ struct SkinnyArgs {
   float* split_ws;
 };
 
+// Several token-major products with the same token count in one launch of the split-K kernel (no K split over
+// workgroups); first_block is filled by the launcher.
+constexpr int kSkinnyMaxGroup = 16;
+struct SkinnyGroupArgs {
+  SkinnyArgs problem[kSkinnyMaxGroup];
+  int first_block[kSkinnyMaxGroup + 1];
+  int count;
+};
+
 enum TileConfig { kTile512x128 = 0, kTile256x128 = 1, kTile128x128 = 2, kTile256x256 = 3, kTile256x128w = 4, kTile512x128t = 5, kTile128x128s = 6, kTile256x64 = 7, kTile256x256w8 = 8, kTile512x128w8 = 9, kTile256x128w8 = 10, kTile128x128w8 = 11, kTile64x128 = 12, kTile128x128k2 = 13, kTile64x128k2 = 14, kTile512x128m16 = 15, kTileAuto = -1 };
 
 hipError_t launch_prepare(const void* a, const void* e, void* prep, int m, int k, int layout, hipStream_t stream);
@@ -71,5 +80,7 @@ hipError_t launch_skinny(SkinnyArgs args, int rows_per_group, hipStream_t stream
 // The linear layer's form of the same kernel: y[t][r] = sum_k W[r][k] x[t][k] + bias[r] for n <= 64 tokens, x and y
 // token-major (x 16-byte aligned).
 hipError_t launch_skinny_tokens(SkinnyArgs args, int rows_per_group, hipStream_t stream);
+// count <= kSkinnyMaxGroup problems of the same form, each with its own weight, x, bias, y, m and k, in one launch.
+hipError_t launch_skinny_group(SkinnyGroupArgs group, int rows_per_group, hipStream_t stream);
 
 }  // namespace onebit
