@@ -60,8 +60,10 @@ void onebit_sparse_matmul(void *a, void *b, void *c, void *d, void *e, int m, in
  * The reordered copy of (a, e) is written on every call to a library-owned workspace kept per device and per
  * stream (grown with a device synchronization when a larger weight arrives; the old buffer is freed, so a HIP graph
  * captured before a larger call on the same stream must be captured again, and a call that would have to grow a
- * buffer while its stream is being captured is refused): calls on different streams may overlap; the prepared form
- * below skips the reorder pass.
+ * buffer while its stream is being captured is refused): calls on different streams may overlap on the GPU. On the
+ * host, a call holds a per-device lock from taking that workspace until both kernels are enqueued, so threads that
+ * submit to one GPU through this entry point take turns (a few microseconds each). The prepared form below skips the
+ * reorder pass and holds the lock only while it looks up its own buffers.
  */
 int onebit_sparse_matmul_ex(const void *a, const void *b, const void *c, void *d, const void *e, int m, int n, int k,
                             float alpha, float beta, int c_dtype, int d_dtype, int meta_layout, void *stream);
