@@ -205,17 +205,22 @@ struct TileShape {
   static_assert(KG == 1 || (KG == 2 && WM * FM <= 4), "the second group's partial tile must fit the stage ring");
 };
 
-// XCD-aware tile order. Workgroup b runs on XCD b % 8, so XCD x is given a contiguous range of a tile list
+// XCD-aware tile order. Workgroup b runs on XCD b % xcds (xcds = 8 on a whole MI355X; the launcher derives it from the
+// device's compute-unit count, so a partitioned GPU keeps the property), so XCD x is given a contiguous range of a tile list
 // that is ordered in blocks of GROUP_M row tiles x 4 column tiles (row tile fastest), blocks running down M inside
 // a strip of 4 column tiles, strips running along N. GROUP_M x 4 = the workgroups resident on one XCD (64 for the
 // four-wavefront tiles with two workgroups per CU; 32 for the tiles with one per CU), which then form one block: every B column
 // panel it streams is shared by GROUP_M workgroups and every A row panel by 4 in that XCD's L2, and the whole
 // range of one XCD covers few column strips, so B is fetched into few L2s.
 template <int GROUP_M>
-__device__ __forceinline__ void tile_of_block(int b, int tiles_m, int tiles_n, int& tm, int& tn) {
+__device__ __forceinline__ void tile_of_block(int b, int tiles_m, int tiles_n, int xcds, int& tm, int& tn) {
   const int total = tiles_m * tiles_n;
-  const int per = total / 8, rem = total % 8;
-  const int x = b % 8, local = b / 8;
+  int per, rem, x, local;
+  if (xcds == 8) {  // the usual case with constant divisors
+    per = total / 8, rem = total % 8, x = b % 8, local = b / 8;
+  } else {
+    per = total / xcds, rem = total % xcds, x = b % xcds, local = b / xcds;
+  }
   const int v = x * per + (x < rem ? x : rem) + local;
   constexpr int STRIP_N = 4;
   const int strip = v / (tiles_m * STRIP_N);
@@ -344,7 +349,7 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
   const int wm = wave_in_group / WN, wn = wave_in_group % WN;
   int tile_m, tile_n;
   // one workgroup per compute unit (eight wavefronts, or four that use all the registers): 32 resident on an XCD
-  tile_of_block<(NW == 8 || FM * FN > 8 ? 8 : 16)>(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  tile_of_block<(NW == 8 || FM * FN > 8 ? 8 : 16)>(blockIdx.x, p.tiles_m, p.tiles_n, p.xcds, tile_m, tile_n);
   const int row0 = tile_m * BM + wm * FM * 32;  // first row of this wavefront
   const int n0 = tile_n * BN;                   // first column of the workgroup
   const int col0 = n0 + wn * FN * 32;           // first column of this wavefront
@@ -952,6 +957,58 @@ __global__ __launch_bounds__(64 * WM * WN * KG, (FM * FN <= 8 ? 2 : 1)) void gem
       __syncthreads();  // every wavefront is done with the stage ring, which becomes the scratch
       constexpr int WCOLS = FN * 32;
       char* scratch = smem + wave * (WCOLS * 128);
+      if constexpr (!M16) if (p.d_f16) {
+        // (measured: 1-5 % off the launch for the 32x32x32 tiles, e.g. 4096 x 4096 with 2048 tokens 37.5 -> 36.7 us; the
+        // 16x16x64 tile, whose single wavefront per SIMD has nothing to hide the conversions behind, is 0.5 % slower
+        // with it and keeps the fp32 form)
+        // fp16 result: the bias is added and the sum rounded in the accumulator layout, where a lane's four registers of
+        // one group are four consecutive rows of its token, i.e. 8 bytes of y. The scratch line of a token then holds its
+        // 32 rows as halves (64 bytes, four 16-byte pieces; piece j of token t stored at position j ^ ((t / 4) % 4), so
+        // that the sixteen lanes that write one slot of sixteen consecutive tokens meet in no bank): half the LDS
+        // traffic of the fp32 form below, same bits (one rounding of sum + bias).
+        typedef float float2v __attribute__((ext_vector_type(2)));
+        typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+        auto packed_rows = [&](const float* x, const float* b4) __attribute__((always_inline)) {
+          const float2v lo = {x[0] + b4[0], x[1] + b4[1]}, hi = {x[2] + b4[2], x[3] + b4[3]};
+          return u32x2_t{__builtin_bit_cast(uint32_t, __builtin_convertvector(lo, half2v)),
+                         __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, half2v))};
+        };
+        // bias of the four rows starting at `row` (a multiple of 4); rows at or past the end are never stored
+        auto bias_rows = [&](int row, float* b4) __attribute__((always_inline)) {
+          if (row < row_limit) bias_vector(row, b4, std::integral_constant<int, 4>{});
+          else b4[0] = b4[1] = b4[2] = b4[3] = 0.f;
+        };
+        auto slot_at = [&](int t, int slot) __attribute__((always_inline)) {  // byte offset of 8-byte slot `slot` of token t
+          return t * 64 + ((((slot >> 1) ^ ((t >> 2) & 3)) << 4) | ((slot & 1) << 3));
+        };
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm) {
+          if (!finishes(fm)) continue;  // the other K group stores this fragment
+          const int row_base = row0 + fm * 32;
+          {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              float b4[4];
+              bias_rows(row_base + 8 * q + 4 * gb, b4);
+#pragma unroll
+              for (int fn = 0; fn < FN; ++fn) {
+                const float x[4] = {acc[fm][fn][4 * q], acc[fm][fn][4 * q + 1], acc[fm][fn][4 * q + 2], acc[fm][fn][4 * q + 3]};
+                *reinterpret_cast<u32x2_t*>(scratch + slot_at(fn * 32 + token_lane, 2 * q + gb)) = packed_rows(x, b4);
+              }
+            }
+          }
+#pragma unroll
+          for (int it = 0; it < WCOLS * 4 / 64; ++it) {
+            const int piece = it * 64 + lane;
+            const int t = piece / 4, j = piece % 4;
+            const int token = col0 + t, row = row_base + 8 * j;
+            const u32x4_t v = *reinterpret_cast<const u32x4_t*>(scratch + slot_at(t, 2 * j));
+            if (token < p.n && row < row_limit)
+              *reinterpret_cast<u32x4_t*>(reinterpret_cast<_Float16*>(d_out) + (size_t)token * p.m + row) = v;
+          }
+        }
+        return;
+      }
 #pragma unroll
       for (int fm = 0; fm < FM; ++fm) {
         if (!finishes(fm)) continue;  // the other K group stores this fragment
@@ -2039,6 +2096,17 @@ static hipError_t launch_gemm_cfg(GemmArgs args, hipStream_t stream) {
     if (st != hipSuccess) return st;
     attr_done[device].store(true, std::memory_order_release);
   }
+  // XCDs of the device as the tile order sees them: gfx950 has 32 compute units per XCD, a whole MI355X eight of them;
+  // a partition of the GPU shows fewer compute units and is served by as many XCDs
+  static std::atomic<int> xcds_of[64] = {};
+  int xcds = xcds_of[device].load(std::memory_order_relaxed);
+  if (xcds <= 0) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) cus = 256;
+    xcds = cus / 32 < 1 ? 1 : (cus / 32 > 8 ? 8 : cus / 32);
+    xcds_of[device].store(xcds, std::memory_order_relaxed);
+  }
+  args.xcds = xcds;
   hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, args.splits), dim3(64 * TS::NW), lds, stream, args);
   return hipGetLastError();
 }

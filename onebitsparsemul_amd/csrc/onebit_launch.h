@@ -15,6 +15,7 @@ struct GemmArgs {
   float alpha, beta;
   int c_f16, d_f16;      // 1: fp16, 0: fp32
   int tiles_m, tiles_n;  // filled by the launcher
+  int xcds;              // filled by the launcher: XCDs the workgroups are dealt over (workgroup b runs on XCD b % xcds)
   int vector_epilogue;   // filled by the launcher: C and D allow 16-byte accesses
   // K split over workgroups (grid.y = splits): split s multiplies the K chunks [s * chunks_per_split, +chunks_per_split)
   // and writes raw fp32 sums to split_ws + s * m * n; a second kernel adds the splits in order and applies the

@@ -237,10 +237,10 @@ def check_reduce(m, n, splits, d_size):
 
 
 # ---------------------------------------------------------------------------------------------------------------
-def tile_of_block(b, tiles_m, tiles_n, group_m):
+def tile_of_block(b, tiles_m, tiles_n, group_m, xcds=8):
     total = tiles_m * tiles_n
-    per, rem = total // 8, total % 8
-    x, local = b % 8, b // 8
+    per, rem = total // xcds, total % xcds
+    x, local = b % xcds, b // xcds
     v = x * per + min(x, rem) + local
     strip = v // (tiles_m * 4)
     strip_w = min(tiles_n - strip * 4, 4)
@@ -272,8 +272,10 @@ def check_gemm(m, n, k, tile, splits, pad_b, tokens=False, b_aligned=True, d_siz
     if tokens:
         assert k * 256 * 2 < (1 << 32)
     # the workgroup -> tile mapping is a bijection
-    seen = {tile_of_block(b, tiles_m, tiles_n, 8 if NW == 8 or FM * FN > 8 else 16) for b in range(tiles_m * tiles_n)}
-    assert seen == {(tm, tn) for tm in range(tiles_m) for tn in range(tiles_n)}
+    # (for every XCD count the launcher can derive: 8 on a whole GPU, fewer on a partition)
+    for xcds in (8, 4, 2, 1):
+        seen = {tile_of_block(b, tiles_m, tiles_n, 8 if NW == 8 or FM * FN > 8 else 16, xcds) for b in range(tiles_m * tiles_n)}
+        assert seen == {(tm, tn) for tm in range(tiles_m) for tn in range(tiles_n)}
     rb_total = m // 32
     corner_tiles = {(0, 0), (tiles_m - 1, 0), (0, tiles_n - 1), (tiles_m - 1, tiles_n - 1), (tiles_m // 2, tiles_n // 2)}
     for split in sorted({0, splits - 1, splits // 2}):
