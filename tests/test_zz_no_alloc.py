@@ -145,3 +145,43 @@ def test_allocating_entry_point_refuses_to_grow_under_capture_and_release_buffer
         _native.matmul_prepared(prep, b, d, m, n, k)  # allocates again after the release
     torch.cuda.synchronize()
     assert np.array_equal(d.cpu().numpy(), ref)
+
+
+def test_weight_cache_refuses_a_miss_under_capture():
+    """A weight that is not in the opt-in cache yet would have to be reordered into newly allocated memory: inside a
+    capture the one-call entry point refuses with a message; after one call outside, the same call is captured, replayed
+    and matches the oracle."""
+    m, n, k = 256, 16, 512
+    a, meta = synthetic.make_weight(m, k, seed=81)
+    bi = synthetic.make_b(k, n, seed=82, kind="int")
+    ad, md, bd = a.cuda(), meta.cuda(), bi.cuda()
+    d = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    ref = oracle.reference_matmul(a.numpy(), bi.numpy(), meta.numpy(), m, n, k, d_dtype=oracle.F32)
+    torch.cuda.synchronize()
+    _native.set_weight_cache(2)
+    try:
+        stream = torch.cuda.Stream()
+        refused = None
+        with torch.cuda.stream(stream):
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                try:
+                    _native.matmul_ex(ad, bd, md, d, m, n, k)
+                except RuntimeError as err:
+                    refused = str(err)
+        assert refused is not None and "being captured" in refused
+        del graph
+        torch.cuda.synchronize()
+        with torch.cuda.stream(stream):
+            _native.matmul_ex(ad, bd, md, d, m, n, k)  # a miss outside the capture: reordered and cached
+            stream.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                _native.matmul_ex(ad, bd, md, d, m, n, k)  # a hit: nothing to allocate
+        d.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(d.cpu().numpy(), ref)
+    finally:
+        _native.set_weight_cache(0)
