@@ -65,9 +65,10 @@ def time_launches(fn, steps, warmup):
     return start.elapsed_time(stop) / steps * 1e-3, wall / steps
 
 
-def time_graph(fn, launches, warmup=20):
+def time_graph(fn, launches, warmup=20, preload_ms=0.0):
     """Average duration of one launch inside a HIP graph of `launches` back-to-back kernel nodes (no host
-    launch overhead between them). The graph is replayed once untimed and once timed."""
+    launch overhead between them). The graph is replayed once untimed (or, with preload_ms, again and again for at least
+    that long, so that the timed replay runs at the clock of a GPU under continuous load) and once timed."""
     import torch
     side = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
@@ -86,8 +87,15 @@ def time_graph(fn, launches, warmup=20):
             for i in range(launches):
                 fn(i)
     torch.cuda.synchronize()
+    t0 = time.perf_counter()
     graph.replay()
     torch.cuda.synchronize()
+    # batches of replays that queue up behind one another (no idle gap inside a batch), each batch about 2 ms of GPU time
+    per_batch = max(1, int(2e-3 / max(time.perf_counter() - t0, 1e-5)))
+    while (time.perf_counter() - t0) * 1e3 < preload_ms:
+        for _ in range(per_batch):
+            graph.replay()
+        torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     graph.replay()
@@ -212,21 +220,14 @@ def cpu_baseline(w, operands, budget_s=12.0, unit="TFLOP/s"):
 
 
 def sustained_rate(fn, flops, load_ms=150.0, launches=60):
-    """The same launch after at least load_ms of continuous load (the GPU raises its clock over the first ~50 ms),
-    timed inside a HIP graph: the rate a long-running job sees, next to `value`, which times the launches right
-    after the warm-up the command line asked for."""
-    import torch
+    """The same launch after at least load_ms of continuous load, timed inside a HIP graph: the rate a long-running job
+    sees. The load is the graph itself replayed back to back, so it is continuous for launches of any length."""
     t0 = time.perf_counter()
-    count = 0
-    while (time.perf_counter() - t0) * 1e3 < load_ms:
-        for _ in range(10):
-            fn(0)
-        torch.cuda.synchronize()
-        count += 10
-    t = time_graph(fn, launches, warmup=10)
+    t = time_graph(fn, launches, warmup=10, preload_ms=load_ms)
     return dict(ms_per_step=t * 1e3, tflops=flops / t / 1e12, frac=flops / t / 1e12 / SMFMAC_PEAK_TFLOPS,
-                preceding_load_ms=(time.perf_counter() - t0) * 1e3, preceding_launches=count, graph_launches=launches,
-                note="HIP-graph timing of the same kernel after >= 150 ms of back-to-back launches (sustained clock)")
+                preceding_load_ms=(time.perf_counter() - t0) * 1e3, graph_launches=launches,
+                note="HIP-graph timing of the same kernel after >= 150 ms of replays of that graph, back to back with no "
+                     "host gap (sustained clock)")
 
 
 def main():
